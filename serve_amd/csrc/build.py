@@ -44,6 +44,10 @@ SOURCES: Dict[str, str] = {
     "attention_mfma": "attention_mfma.hip",
     "membench": "membench.hip",
     "blaslt": "blaslt.hip",
+    "sublayer": "sublayer.hip",
+    "delta_rule": "delta_rule.hip",
+    "latent": "latent.hip",
+    "moe": "moe.hip",
 }
 # what a library is linked with beside the HIP runtime
 LINK: Dict[str, List[str]] = {"blaslt.hip": ["-lhipblaslt"]}

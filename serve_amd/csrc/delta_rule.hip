@@ -1,0 +1,305 @@
+// The gated delta rule: a linear-attention mixer with one fp32 state matrix per head and request.
+//
+//   per head and token:  S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+//
+// q, k [dk] and v [dv] come from projections that pass a short causal convolution over time (one
+// filter per channel, `taps` taps, the last tap on the current token) and silu; q and k are made unit
+// vectors per head (q also times dk^-1/2); beta = sigmoid(b); g = exp(-exp(A_log) softplus(a + dt_bias)).
+// A request's state row holds S of every head ([H, dk, dv]) and behind it the last taps - 1 inputs of
+// the convolution ([taps - 1, C], oldest first), all fp32.  Everything here is fp32 arithmetic; only the
+// projections' storage type is templated.
+//
+// Four kernels a step: (1) convolution + silu + unit vectors + beta and g for every token, in
+// parallel; (2) the convolution's new state; (3) the recurrence, a workgroup per (segment, head, tile
+// of columns of S), token after token; (4) the read-out's norm per head times the output gate.
+#include "common.h"
+
+#define DR_MAX_TAPS 16
+
+__device__ __forceinline__ float silu_f(float z) { return z / (1.f + expf(-z)); }
+__device__ __forceinline__ float softplus_f(float z) { return fmaxf(z, 0.f) + log1pf(expf(-fabsf(z))); }
+
+// ---------------------------------------------------------------------------------------------
+// (1) z [T, zs]: columns [q: Hk dk | k: Hk dk | v: H dv | ...]; the first C = 2 Hk dk + H dv of
+// them are the convolution's channels.  grid (T, 2 Hk + H + 1): a workgroup of 64 threads per token
+// and head of q, k or v, and one for the token's beta and g.
+// ---------------------------------------------------------------------------------------------
+template <typename TA>
+__global__ __launch_bounds__(64) void delta_prepare_kernel(
+    const TA* __restrict__ z, int zs, const float* __restrict__ conv_w, const float* __restrict__ state,
+    size_t state_stride, size_t conv_off, const float* __restrict__ ba, const float* __restrict__ A_log,
+    const float* __restrict__ dt_bias, const int* __restrict__ seg_of_token, const int* __restrict__ cu_q,
+    const int* __restrict__ state_slots, float* __restrict__ qn, float* __restrict__ kn, float* __restrict__ vc,
+    float* __restrict__ beta, float* __restrict__ decay, int H, int Hk, int dk, int dv, int taps) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x;
+  const int u = blockIdx.y;
+  if (u == 2 * Hk + H) {
+    for (int h = threadIdx.x; h < H; h += blockDim.x) {
+      const float b = ba[(size_t)t * 2 * H + h];
+      const float a = ba[(size_t)t * 2 * H + H + h];
+      beta[(size_t)t * H + h] = 1.f / (1.f + expf(-b));
+      decay[(size_t)t * H + h] = expf(-expf(A_log[h]) * softplus_f(a + dt_bias[h]));
+    }
+    return;
+  }
+  const int seg = seg_of_token[t];
+  const int t0 = cu_q[seg];
+  const int slot = state_slots[seg];
+  const int C = 2 * Hk * dk + H * dv;
+  int c0, n, kind;
+  float* dst;
+  if (u < Hk) { kind = 0; n = dk; c0 = u * dk; dst = qn + ((size_t)t * Hk + u) * dk; }
+  else if (u < 2 * Hk) { kind = 1; n = dk; c0 = Hk * dk + (u - Hk) * dk; dst = kn + ((size_t)t * Hk + (u - Hk)) * dk; }
+  else { kind = 2; n = dv; c0 = 2 * Hk * dk + (u - 2 * Hk) * dv; dst = vc + ((size_t)t * H + (u - 2 * Hk)) * dv; }
+  const float* cs = slot >= 0 ? state + (size_t)slot * state_stride + conv_off : nullptr;
+  float vals[4];          // n <= 256
+  float ss = 0.f;
+#pragma unroll
+  for (int m = 0; m < 4; ++m) {
+    const int i = threadIdx.x + m * 64;
+    float y = 0.f;
+    if (i < n) {
+      const int c = c0 + i;
+      float acc = 0.f;
+      for (int j = 0; j < taps; ++j) {
+        const int tp = t - (taps - 1 - j);
+        float xv;
+        if (tp >= t0) xv = to_float(z[(size_t)tp * zs + c]);
+        else xv = cs ? cs[(size_t)(taps - 1 + tp - t0) * C + c] : 0.f;
+        acc += conv_w[(size_t)c * taps + j] * xv;
+      }
+      y = silu_f(acc);
+    }
+    vals[m] = y;
+    ss += y * y;
+  }
+  float scale = 1.f;
+  if (kind != 2) {
+    ss = block_sum(ss, scratch);
+    scale = 1.f / sqrtf(ss + 1e-6f);
+    if (kind == 0) scale *= 1.f / sqrtf((float)dk);
+  }
+#pragma unroll
+  for (int m = 0; m < 4; ++m) {
+    const int i = threadIdx.x + m * 64;
+    if (i < n) dst[i] = vals[m] * scale;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// (2) the last taps - 1 inputs of every channel after the step: from the step's own tokens, and
+// from the old state where the segment brought fewer than taps - 1.  grid (B, ceil(C / 256)).
+// ---------------------------------------------------------------------------------------------
+template <typename TA>
+__global__ __launch_bounds__(256) void delta_conv_state_kernel(
+    const TA* __restrict__ z, int zs, float* __restrict__ state, size_t state_stride, size_t conv_off,
+    const int* __restrict__ cu_q, const int* __restrict__ state_slots, int C, int taps) {
+  const int seg = blockIdx.x;
+  const int slot = state_slots[seg];
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (slot < 0 || c >= C) return;
+  const int t0 = cu_q[seg], n = cu_q[seg + 1] - t0;
+  float* cs = state + (size_t)slot * state_stride + conv_off;
+  float nv[DR_MAX_TAPS - 1];
+#pragma unroll
+  for (int i = 0; i < DR_MAX_TAPS - 1; ++i) {
+    if (i < taps - 1) {
+      const int li = n - (taps - 1) + i;
+      nv[i] = li >= 0 ? to_float(z[(size_t)(t0 + li) * zs + c]) : cs[(size_t)(i + n) * C + c];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < DR_MAX_TAPS - 1; ++i)
+    if (i < taps - 1) cs[(size_t)i * C + c] = nv[i];
+}
+
+// ---------------------------------------------------------------------------------------------
+// (3) the recurrence.  grid (ceil(dv / COLS), H, B); a wave holds 16 columns of S, each cut in four
+// parts along dk (a thread keeps RPT rows of one column in registers), so that S^T k and S^T q are
+// sums inside a thread plus two exchanges between neighbouring lanes.  The tokens of a segment come
+// through LDS in chunks of CH; a segment's state is read once and written once.
+// ---------------------------------------------------------------------------------------------
+#define DR_CH 16
+
+template <int RPT>
+__global__ __launch_bounds__(256) void delta_recurrence_kernel(
+    const float* __restrict__ qn, const float* __restrict__ kn, const float* __restrict__ vc,
+    const float* __restrict__ beta, const float* __restrict__ decay, float* __restrict__ state,
+    size_t state_stride, const int* __restrict__ cu_q, const int* __restrict__ state_slots,
+    float* __restrict__ o, int H, int Hk, int dk, int dv) {
+  constexpr int PAD = RPT + 4;           // a part's rows in LDS, padded so that the four parts lie in other banks
+  constexpr int ROW = 4 * PAD;
+  __shared__ __attribute__((aligned(16))) float sq[DR_CH][ROW];
+  __shared__ __attribute__((aligned(16))) float sk[DR_CH][ROW];
+  __shared__ float sv[DR_CH][64];
+  __shared__ float sb[DR_CH], sg[DR_CH];
+  const int cols = blockDim.x >> 2;
+  const int cl = threadIdx.x >> 2, r = threadIdx.x & 3;
+  const int j = blockIdx.x * cols + cl;
+  const int h = blockIdx.y, seg = blockIdx.z;
+  const int hk = h / (H / Hk);
+  const bool active = j < dv;
+  const int slot = state_slots[seg];
+  const int t0 = cu_q[seg], n = cu_q[seg + 1] - t0;
+  float* st = slot >= 0 ? state + (size_t)slot * state_stride + (size_t)h * dk * dv : nullptr;
+  float S[RPT];
+#pragma unroll
+  for (int ii = 0; ii < RPT; ++ii) {
+    const int i = r * RPT + ii;
+    S[ii] = (st && active && i < dk) ? st[(size_t)i * dv + j] : 0.f;
+  }
+  for (int c0 = 0; c0 < n; c0 += DR_CH) {
+    const int m = min(DR_CH, n - c0);
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < DR_CH * 4 * RPT; idx += blockDim.x) {
+      const int tt = idx / (4 * RPT), i = idx - tt * (4 * RPT);
+      const int pos = (i / RPT) * PAD + (i % RPT);
+      const bool in = tt < m && i < dk;
+      const size_t src = ((size_t)(t0 + c0 + tt) * Hk + hk) * dk + i;
+      sq[tt][pos] = in ? qn[src] : 0.f;
+      sk[tt][pos] = in ? kn[src] : 0.f;
+    }
+    for (int idx = threadIdx.x; idx < DR_CH * cols; idx += blockDim.x) {
+      const int tt = idx / cols, c = idx - tt * cols;
+      const int jj = blockIdx.x * cols + c;
+      sv[tt][c] = (tt < m && jj < dv) ? vc[((size_t)(t0 + c0 + tt) * H + h) * dv + jj] : 0.f;
+    }
+    if (threadIdx.x < DR_CH) {
+      const int tt = threadIdx.x;
+      sb[tt] = tt < m ? beta[(size_t)(t0 + c0 + tt) * H + h] : 0.f;
+      sg[tt] = tt < m ? decay[(size_t)(t0 + c0 + tt) * H + h] : 1.f;
+    }
+    __syncthreads();
+    for (int tt = 0; tt < m; ++tt) {
+      const float g = sg[tt], b = sb[tt];
+      const float* kr = &sk[tt][r * PAD];
+      const float* qr = &sq[tt][r * PAD];
+      float kv = 0.f;
+#pragma unroll
+      for (int ii = 0; ii < RPT; ++ii) {
+        S[ii] *= g;
+        kv += S[ii] * kr[ii];
+      }
+      kv += __shfl_xor(kv, 1, SA_WAVE);
+      kv += __shfl_xor(kv, 2, SA_WAVE);
+      const float u = b * (sv[tt][cl] - kv);
+      float oo = 0.f;
+#pragma unroll
+      for (int ii = 0; ii < RPT; ++ii) {
+        S[ii] += kr[ii] * u;
+        oo += S[ii] * qr[ii];
+      }
+      oo += __shfl_xor(oo, 1, SA_WAVE);
+      oo += __shfl_xor(oo, 2, SA_WAVE);
+      if (r == 0 && active) o[((size_t)(t0 + c0 + tt) * H + h) * dv + j] = oo;
+    }
+  }
+  if (st && active) {
+#pragma unroll
+    for (int ii = 0; ii < RPT; ++ii) {
+      const int i = r * RPT + ii;
+      if (i < dk) st[(size_t)i * dv + j] = S[ii];
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// (4) y[t, h, :] = o[t, h, :] / sqrt(mean(o^2) + eps) * w * silu(gate[t, h, :]); gate is a block of
+// columns of z.  A wave per (token, head).
+// ---------------------------------------------------------------------------------------------
+template <typename TA>
+__global__ __launch_bounds__(256) void delta_gated_norm_kernel(const float* __restrict__ o, const TA* __restrict__ z,
+                                                               int zs, int gate_col, const float* __restrict__ w,
+                                                               TA* __restrict__ y, float eps, int TH, int H, int dv) {
+  const int p = blockIdx.x * (blockDim.x / SA_WAVE) + threadIdx.x / SA_WAVE;
+  if (p >= TH) return;
+  const int lane = threadIdx.x & (SA_WAVE - 1);
+  const int t = p / H, h = p - t * H;
+  const float* op = o + (size_t)p * dv;
+  float ss = 0.f;
+  for (int i = lane; i < dv; i += SA_WAVE) ss += op[i] * op[i];
+  ss = wave_sum(ss);
+  const float rs = 1.f / sqrtf(ss / (float)dv + eps);
+  const TA* gp = z + (size_t)t * zs + gate_col + (size_t)h * dv;
+  for (int i = lane; i < dv; i += SA_WAVE)
+    y[(size_t)p * dv + i] = from_float<TA>(((op[i] * rs) * w[i]) * silu_f(to_float(gp[i])));
+}
+
+// ---------------------------------------------------------------------------------------------
+// One call runs the four kernels.  z: the fused projections [T, zs] = [q | k | v | gate | ...];
+// ba fp32 [T, 2 H] (b then a); work: fp32 scratch of T (2 Hk dk + 2 H dv + 2 H) floats; y [T, H dv].
+// ---------------------------------------------------------------------------------------------
+extern "C" long long sa_delta_rule_work_floats(int T, int H, int Hk, int dk, int dv) {
+  return (long long)T * (2LL * Hk * dk + 2LL * H * dv + 2LL * H);
+}
+
+extern "C" int sa_delta_rule(const void* z, int act_dtype, int zs, const float* conv_w, const float* ba,
+                             const float* A_log, const float* dt_bias, const float* norm_w, float* state,
+                             long long state_stride, const int* seg_of_token, const int* cu_q,
+                             const int* state_slots, float* work, void* y, float eps, int T, int B, int H, int Hk,
+                             int dk, int dv, int taps, hipStream_t stream) {
+  if (T <= 0 || B <= 0) return 0;
+  if (H <= 0 || Hk <= 0 || H % Hk || dk <= 0 || dk > 256 || dv <= 0 || dv > 256 || taps < 1 || taps > DR_MAX_TAPS)
+    return SA_ERR_ARG;
+  if (B > 65535 || H > 65535 || 2 * Hk + H + 1 > 65535) return SA_ERR_ARG;
+  const int C = 2 * Hk * dk + H * dv;
+  if (zs < C + H * dv) return SA_ERR_ARG;
+  const size_t conv_off = (size_t)H * dk * dv;
+  if ((size_t)state_stride < conv_off + (size_t)(taps - 1) * C) return SA_ERR_ARG;
+  float* qn = work;
+  float* kn = qn + (size_t)T * Hk * dk;
+  float* vc = kn + (size_t)T * Hk * dk;
+  float* o = vc + (size_t)T * H * dv;
+  float* beta = o + (size_t)T * H * dv;
+  float* decay = beta + (size_t)T * H;
+  {
+    dim3 grid(T, 2 * Hk + H + 1), block(64);
+    if (act_dtype == SA_F32)
+      hipLaunchKernelGGL(delta_prepare_kernel<float>, grid, block, 0, stream, (const float*)z, zs, conv_w, state,
+                         (size_t)state_stride, conv_off, ba, A_log, dt_bias, seg_of_token, cu_q, state_slots, qn, kn,
+                         vc, beta, decay, H, Hk, dk, dv, taps);
+    else if (act_dtype == SA_BF16)
+      hipLaunchKernelGGL(delta_prepare_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)z, zs, conv_w, state,
+                         (size_t)state_stride, conv_off, ba, A_log, dt_bias, seg_of_token, cu_q, state_slots, qn, kn,
+                         vc, beta, decay, H, Hk, dk, dv, taps);
+    else return SA_ERR_UNSUPPORTED;
+    SA_LAUNCH_CHECK();
+  }
+  if (taps > 1) {
+    dim3 grid(B, (C + 255) / 256), block(256);
+    if (act_dtype == SA_F32)
+      hipLaunchKernelGGL(delta_conv_state_kernel<float>, grid, block, 0, stream, (const float*)z, zs, state,
+                         (size_t)state_stride, conv_off, cu_q, state_slots, C, taps);
+    else
+      hipLaunchKernelGGL(delta_conv_state_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)z, zs, state,
+                         (size_t)state_stride, conv_off, cu_q, state_slots, C, taps);
+    SA_LAUNCH_CHECK();
+  }
+  {
+    const int waves = dv >= 64 ? 4 : (dv + 15) / 16;
+    const int cols = 16 * waves;
+    dim3 grid((dv + cols - 1) / cols, H, B), block(64 * waves);
+#define GO(RPT)                                                                                                 \
+  hipLaunchKernelGGL(delta_recurrence_kernel<RPT>, grid, block, 0, stream, qn, kn, vc, beta, decay, state,      \
+                     (size_t)state_stride, cu_q, state_slots, o, H, Hk, dk, dv)
+    if (dk <= 64) GO(16);
+    else if (dk <= 128) GO(32);
+    else GO(64);
+#undef GO
+    SA_LAUNCH_CHECK();
+  }
+  {
+    const long long TH = (long long)T * H;
+    if (TH > 0x7fffffffLL) return SA_ERR_ARG;
+    dim3 grid((unsigned)((TH + 3) / 4)), block(256);
+    if (act_dtype == SA_F32)
+      hipLaunchKernelGGL(delta_gated_norm_kernel<float>, grid, block, 0, stream, o, (const float*)z, zs, C, norm_w,
+                         (float*)y, eps, (int)TH, H, dv);
+    else
+      hipLaunchKernelGGL(delta_gated_norm_kernel<bf16_t>, grid, block, 0, stream, o, (const bf16_t*)z, zs, C, norm_w,
+                         (bf16_t*)y, eps, (int)TH, H, dv);
+    SA_LAUNCH_CHECK();
+  }
+  return 0;
+}

@@ -1,0 +1,296 @@
+// Routed experts: every token takes the `top` experts with the largest router logits, weighted by the
+// softmax over those logits alone; an expert is down(silu(gate x) * up x).
+//
+// Nothing is read back to the host: the tokens are grouped by expert on the device, and the
+// products run over a list of (expert, rows) tiles that is built there, from a grid sized for
+// the worst case whose surplus workgroups leave at once.
+//
+//   route     logits fp32 [T, ldz] -> ids int32 [T, top], weights fp32 [T, top]
+//   group     ids -> offsets[E + 1], perm[T top] (row of the grouped order -> t * top + k),
+//             tile_expert[], tile_row0[], num_tiles
+//   gate_up   act[row, :] = silu(Wg_e x) * (Wu_e x),  x = h[perm[row] / top]
+//   down      yk[perm[row], :] = Wd_e act[row, :]          (fp32)
+//   combine   y[t, :] = sum_k weights[t, k] yk[t top + k, :]  (+ sigmoid(sg[t]) * shared[t, :])
+//
+// Products: fp32 sums on the vector ALU over LDS tiles, storage types templated.
+#include "common.h"
+
+#define MOE_TM 32
+#define MOE_TN 64
+#define MOE_TK 32
+
+// ---------------------------------------------------------------------------------------------
+// route: a wave per token.  Ties go to the lower index.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int ldz, int* __restrict__ ids,
+                                                        float* __restrict__ wts, int T, int E, int top) {
+  const int t = blockIdx.x * (blockDim.x / SA_WAVE) + threadIdx.x / SA_WAVE;
+  if (t >= T) return;
+  const int lane = threadIdx.x & (SA_WAVE - 1);
+  const float* z = logits + (size_t)t * ldz;
+  float prev_v = INFINITY;
+  int prev_i = -1;
+  float first = 0.f, sum = 0.f;
+  for (int k = 0; k < top; ++k) {
+    // the largest logit that comes after (prev_v, prev_i) in the order (value descending, index ascending)
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int e = lane; e < E; e += SA_WAVE) {
+      const float v = z[e];
+      const bool after = v < prev_v || (v == prev_v && e > prev_i);
+      if (after && (v > bv || (v == bv && e < bi))) { bv = v; bi = e; }
+    }
+#pragma unroll
+    for (int o = SA_WAVE / 2; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, SA_WAVE);
+      const int oi = __shfl_xor(bi, o, SA_WAVE);
+      if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    }
+    if (k == 0) first = bv;
+    const float p = expf(bv - first);
+    sum += p;
+    if (lane == 0) {
+      ids[(size_t)t * top + k] = bi;
+      wts[(size_t)t * top + k] = p;
+    }
+    prev_v = bv;
+    prev_i = bi;
+  }
+  if (lane == 0)
+    for (int k = 0; k < top; ++k) wts[(size_t)t * top + k] /= sum;
+}
+
+// ---------------------------------------------------------------------------------------------
+// group: one workgroup.  Counts per expert, their running sum, the tiles, then every (token, k)
+// takes the next free row of its expert (the order inside an expert does not matter: a row's sums
+// do not depend on its place).
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__ ids, int n, int E,
+                                                         int* __restrict__ offsets, int* __restrict__ cursor,
+                                                         int* __restrict__ perm, int* __restrict__ tile_expert,
+                                                         int* __restrict__ tile_row0, int* __restrict__ num_tiles) {
+  for (int e = threadIdx.x; e < E; e += blockDim.x) cursor[e] = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < n; i += blockDim.x) atomicAdd(&cursor[ids[i]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0, tiles = 0;
+    for (int e = 0; e < E; ++e) {
+      const int c = cursor[e];
+      offsets[e] = run;
+      for (int r0 = 0; r0 < c; r0 += MOE_TM) {
+        tile_expert[tiles] = e;
+        tile_row0[tiles] = run + r0;
+        ++tiles;
+      }
+      cursor[e] = run;
+      run += c;
+    }
+    offsets[E] = run;
+    *num_tiles = tiles;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < n; i += blockDim.x) perm[atomicAdd(&cursor[ids[i]], 1)] = i;
+}
+
+// ---------------------------------------------------------------------------------------------
+// The tile product: C[TM x TN] = A[TM x K] . W[TN x K]^T, both contiguous along K.  256 threads,
+// thread (ty, tx) = (tid / 16, tid % 16) owns rows ty, ty + 16 and columns tx + 16 c, c < 4.
+// ---------------------------------------------------------------------------------------------
+template <typename TA, typename TW, bool DUAL>
+__device__ __forceinline__ void tile_product(const TA* __restrict__ A, const int* a_row_index,
+                                             int a_stride, int rows, const TW* __restrict__ W0,
+                                             const TW* __restrict__ W1, int n0, int N, int K, float acc0[2][4],
+                                             float acc1[2][4], float (*sa)[MOE_TM + 1], float (*sw0)[MOE_TN + 1],
+                                             float (*sw1)[MOE_TN + 1]) {
+  const int tid = threadIdx.x;
+  const int ty = tid >> 4, tx = tid & 15;
+  for (int k0 = 0; k0 < K; k0 += MOE_TK) {
+    __syncthreads();
+    for (int idx = tid; idx < MOE_TM * MOE_TK; idx += 256) {
+      const int r = idx / MOE_TK, k = idx - r * MOE_TK;
+      float v = 0.f;
+      if (r < rows && k0 + k < K) v = to_float(A[(size_t)a_row_index[r] * a_stride + k0 + k]);
+      sa[k][r] = v;
+    }
+    for (int idx = tid; idx < MOE_TN * MOE_TK; idx += 256) {
+      const int c = idx / MOE_TK, k = idx - c * MOE_TK;
+      const bool in = n0 + c < N && k0 + k < K;
+      sw0[k][c] = in ? to_float(W0[(size_t)(n0 + c) * K + k0 + k]) : 0.f;
+      if (DUAL) sw1[k][c] = in ? to_float(W1[(size_t)(n0 + c) * K + k0 + k]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll 8
+    for (int k = 0; k < MOE_TK; ++k) {
+      const float a0 = sa[k][ty], a1 = sa[k][ty + 16];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const float w0 = sw0[k][tx + 16 * c];
+        acc0[0][c] += a0 * w0;
+        acc0[1][c] += a1 * w0;
+        if (DUAL) {
+          const float w1 = sw1[k][tx + 16 * c];
+          acc1[0][c] += a0 * w1;
+          acc1[1][c] += a1 * w1;
+        }
+      }
+    }
+  }
+}
+
+// gate_up: grid (max tiles, ceil(F / TN)).  Wg, Wu [E, F, d]; h [T, d]; act [T top, F] in grouped order.
+template <typename TA>
+__global__ __launch_bounds__(256) void moe_gate_up_kernel(const TA* __restrict__ h, const TA* __restrict__ Wg,
+                                                          const TA* __restrict__ Wu, const int* __restrict__ offsets,
+                                                          const int* __restrict__ perm, const int* __restrict__ tile_expert,
+                                                          const int* __restrict__ tile_row0, const int* __restrict__ num_tiles,
+                                                          TA* __restrict__ act, int top, int d, int F) {
+  __shared__ float sa[MOE_TK][MOE_TM + 1];
+  __shared__ float sw0[MOE_TK][MOE_TN + 1];
+  __shared__ float sw1[MOE_TK][MOE_TN + 1];
+  __shared__ int rowidx[MOE_TM];
+  const int tile = blockIdx.x;
+  if (tile >= *num_tiles) return;
+  const int e = tile_expert[tile], row0 = tile_row0[tile];
+  const int rows = min(MOE_TM, offsets[e + 1] - row0);
+  if (threadIdx.x < MOE_TM) rowidx[threadIdx.x] = threadIdx.x < rows ? perm[row0 + threadIdx.x] / top : 0;
+  const int n0 = blockIdx.y * MOE_TN;
+  float g[2][4] = {}, u[2][4] = {};
+  tile_product<TA, TA, true>(h, rowidx, d, rows, Wg + (size_t)e * F * d, Wu + (size_t)e * F * d, n0, F, d, g, u,
+                             sa, sw0, sw1);
+  const int ty = threadIdx.x >> 4, tx = threadIdx.x & 15;
+#pragma unroll
+  for (int rr = 0; rr < 2; ++rr) {
+    const int r = ty + 16 * rr;
+    if (r >= rows) continue;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int n = n0 + tx + 16 * c;
+      if (n < F) {
+        const float gv = g[rr][c];
+        act[(size_t)(row0 + r) * F + n] = from_float<TA>((gv / (1.f + expf(-gv))) * u[rr][c]);
+      }
+    }
+  }
+}
+
+// down: grid (max tiles, ceil(d / TN)).  Wd [E, d, F]; act [T top, F] grouped; yk fp32 [T top, d] by (t, k).
+template <typename TA>
+__global__ __launch_bounds__(256) void moe_down_kernel(const TA* __restrict__ act, const TA* __restrict__ Wd,
+                                                       const int* __restrict__ offsets, const int* __restrict__ perm,
+                                                       const int* __restrict__ tile_expert, const int* __restrict__ tile_row0,
+                                                       const int* __restrict__ num_tiles, float* __restrict__ yk, int d,
+                                                       int F) {
+  __shared__ float sa[MOE_TK][MOE_TM + 1];
+  __shared__ float sw0[MOE_TK][MOE_TN + 1];
+  __shared__ int rowidx[MOE_TM];
+  const int tile = blockIdx.x;
+  if (tile >= *num_tiles) return;
+  const int e = tile_expert[tile], row0 = tile_row0[tile];
+  const int rows = min(MOE_TM, offsets[e + 1] - row0);
+  if (threadIdx.x < MOE_TM) rowidx[threadIdx.x] = threadIdx.x < rows ? row0 + threadIdx.x : 0;
+  const int n0 = blockIdx.y * MOE_TN;
+  float acc[2][4] = {}, none[2][4];
+  tile_product<TA, TA, false>(act, rowidx, F, rows, Wd + (size_t)e * d * F, nullptr, n0, d, F, acc, none, sa,
+                              sw0, nullptr);
+  const int ty = threadIdx.x >> 4, tx = threadIdx.x & 15;
+#pragma unroll
+  for (int rr = 0; rr < 2; ++rr) {
+    const int r = ty + 16 * rr;
+    if (r >= rows) continue;
+    const size_t dst = (size_t)perm[row0 + r] * d;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int n = n0 + tx + 16 * c;
+      if (n < d) yk[dst + n] = acc[rr][c];
+    }
+  }
+}
+
+// combine: grid (T).  shared: [parts, T, d] (TS), or null; sg: logits fp32, row stride ldz (null: no gate).
+template <typename TS>
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ yk, const float* __restrict__ wts,
+                                                          const TS* __restrict__ shared, int parts, size_t part_stride,
+                                                          const float* __restrict__ sg, int ldz, float* __restrict__ y,
+                                                          int top, int d) {
+  const int t = blockIdx.x;
+  float gate = 1.f;
+  if (shared && sg) gate = 1.f / (1.f + expf(-sg[(size_t)t * ldz]));
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    float v = 0.f;
+    for (int k = 0; k < top; ++k) v += wts[(size_t)t * top + k] * yk[((size_t)t * top + k) * d + i];
+    if (shared) {
+      float s = 0.f;
+      for (int p = 0; p < parts; ++p) s += to_float(shared[p * part_stride + (size_t)t * d + i]);
+      v += gate * s;
+    }
+    y[(size_t)t * d + i] = v;
+  }
+}
+
+extern "C" int sa_moe_max_tiles(int rows, int E) { return (rows + MOE_TM - 1) / MOE_TM + E; }
+
+extern "C" int sa_moe_route(const float* logits, int ldz, int* ids, float* wts, int T, int E, int top,
+                            hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (E <= 0 || top <= 0 || top > E || ldz < E) return SA_ERR_ARG;
+  dim3 grid((T + 3) / 4), block(256);
+  hipLaunchKernelGGL(moe_route_kernel, grid, block, 0, stream, logits, ldz, ids, wts, T, E, top);
+  SA_LAUNCH_CHECK();
+  return 0;
+}
+
+// ints: scratch of (E + 1) + E + n + 2 max_tiles + 1 int32 (offsets, cursor, perm, tile_expert, tile_row0, num_tiles)
+extern "C" int sa_moe_experts(const void* h, int act_dtype, const int* ids, const void* Wg, const void* Wu,
+                              const void* Wd, int* ints, void* act, float* yk, int T, int top, int E, int d, int F,
+                              hipStream_t stream) {
+  if (T <= 0) return 0;
+  const long long n = (long long)T * top;
+  if (E <= 0 || top <= 0 || d <= 0 || F <= 0 || n > 0x3fffffffLL) return SA_ERR_ARG;
+  const int max_tiles = sa_moe_max_tiles((int)n, E);
+  int* offsets = ints;
+  int* cursor = offsets + E + 1;
+  int* perm = cursor + E;
+  int* tile_expert = perm + n;
+  int* tile_row0 = tile_expert + max_tiles;
+  int* num_tiles = tile_row0 + max_tiles;
+  hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), 0, stream, ids, (int)n, E, offsets, cursor, perm,
+                     tile_expert, tile_row0, num_tiles);
+  SA_LAUNCH_CHECK();
+  dim3 g1(max_tiles, (F + MOE_TN - 1) / MOE_TN), g2(max_tiles, (d + MOE_TN - 1) / MOE_TN), block(256);
+  if (g1.y > 65535 || g2.y > 65535) return SA_ERR_ARG;
+  if (act_dtype == SA_F32) {
+    hipLaunchKernelGGL(moe_gate_up_kernel<float>, g1, block, 0, stream, (const float*)h, (const float*)Wg,
+                       (const float*)Wu, offsets, perm, tile_expert, tile_row0, num_tiles, (float*)act, top, d, F);
+    SA_LAUNCH_CHECK();
+    hipLaunchKernelGGL(moe_down_kernel<float>, g2, block, 0, stream, (const float*)act, (const float*)Wd, offsets, perm,
+                       tile_expert, tile_row0, num_tiles, yk, d, F);
+  } else if (act_dtype == SA_BF16) {
+    hipLaunchKernelGGL(moe_gate_up_kernel<bf16_t>, g1, block, 0, stream, (const bf16_t*)h, (const bf16_t*)Wg,
+                       (const bf16_t*)Wu, offsets, perm, tile_expert, tile_row0, num_tiles, (bf16_t*)act, top, d, F);
+    SA_LAUNCH_CHECK();
+    hipLaunchKernelGGL(moe_down_kernel<bf16_t>, g2, block, 0, stream, (const bf16_t*)act, (const bf16_t*)Wd, offsets,
+                       perm, tile_expert, tile_row0, num_tiles, yk, d, F);
+  } else {
+    return SA_ERR_UNSUPPORTED;
+  }
+  SA_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int sa_moe_combine(const float* yk, const float* wts, const void* shared, int shared_dtype, int parts,
+                              const float* sg, int ldz, float* y, int T, int top, int d, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (top <= 0 || d <= 0 || parts < 1) return SA_ERR_ARG;
+  const size_t part_stride = (size_t)T * d;
+  dim3 grid(T), block(d >= 256 ? 256 : 64);
+  if (!shared || shared_dtype == SA_F32)
+    hipLaunchKernelGGL(moe_combine_kernel<float>, grid, block, 0, stream, yk, wts, (const float*)shared, parts,
+                       part_stride, sg, ldz, y, top, d);
+  else if (shared_dtype == SA_BF16 && parts == 1)
+    hipLaunchKernelGGL(moe_combine_kernel<bf16_t>, grid, block, 0, stream, yk, wts, (const bf16_t*)shared, parts,
+                       part_stride, sg, ldz, y, top, d);
+  else return SA_ERR_UNSUPPORTED;
+  SA_LAUNCH_CHECK();
+  return 0;
+}

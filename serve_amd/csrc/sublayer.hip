@@ -1,0 +1,120 @@
+// Elementwise kernels of layers whose norm sits on the sublayer's output:
+//   x <- x + s * N(y),  N(y) = y / sqrt(mean(y^2) + eps) * w      (x: fp32 residual stream)
+// and of feed-forwards with a plain activation between two products.  fp32 arithmetic; the
+// storage types of activations are templated.
+#include "common.h"
+
+// ---------------------------------------------------------------------------------------------
+// x[t] += (N(y[t]) * w) * s, and h[t] = x[t] in the activation dtype for the sublayer that reads
+// the stream next.  y is [T, d] in the activation dtype or fp32, or fp32 [parts, T, d] partial
+// sums that are added in order (a product whose inner dimension was cut across workgroups, the
+// experts of a token).  y == nullptr: only the copy h = x is made.  h == nullptr: no copy.
+// One workgroup a row; a thread keeps up to VMAX of its values between the two passes, the rest
+// is read again.
+// ---------------------------------------------------------------------------------------------
+template <typename TA, typename TD>
+__global__ __launch_bounds__(256) void output_norm_add_kernel(float* __restrict__ x, const TD* __restrict__ y,
+                                                              int parts, size_t part_stride,
+                                                              const float* __restrict__ w,
+                                                              const float* __restrict__ s, TA* __restrict__ h,
+                                                              float eps, int d) {
+  __shared__ float scratch[16];
+  constexpr int VMAX = 8;
+  const int t = blockIdx.x;
+  float* xr = x + (size_t)t * d;
+  TA* hr = h ? h + (size_t)t * d : nullptr;
+  if (!y) {
+    if (hr)
+      for (int i = threadIdx.x; i < d; i += blockDim.x) hr[i] = from_float<TA>(xr[i]);
+    return;
+  }
+  const TD* yr = y + (size_t)t * d;
+  float keep[VMAX];
+  float ss = 0.f;
+  const int bd = blockDim.x;
+#pragma unroll
+  for (int n = 0; n < VMAX; ++n) {
+    const int i = threadIdx.x + n * bd;
+    float v = 0.f;
+    if (i < d)
+      for (int p = 0; p < parts; ++p) v += to_float(yr[p * part_stride + i]);
+    keep[n] = v;
+    ss += v * v;
+  }
+  for (int i = threadIdx.x + VMAX * bd; i < d; i += bd) {
+    float v = 0.f;
+    for (int p = 0; p < parts; ++p) v += to_float(yr[p * part_stride + i]);
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float rs = 1.0f / sqrtf(ss / (float)d + eps);
+#pragma unroll
+  for (int n = 0; n < VMAX; ++n) {
+    const int i = threadIdx.x + n * bd;
+    if (i < d) {
+      const float nx = xr[i] + ((keep[n] * rs) * w[i]) * s[i];
+      xr[i] = nx;
+      if (hr) hr[i] = from_float<TA>(nx);
+    }
+  }
+  for (int i = threadIdx.x + VMAX * bd; i < d; i += bd) {
+    float v = 0.f;
+    for (int p = 0; p < parts; ++p) v += to_float(yr[p * part_stride + i]);
+    const float nx = xr[i] + ((v * rs) * w[i]) * s[i];
+    xr[i] = nx;
+    if (hr) hr[i] = from_float<TA>(nx);
+  }
+}
+
+extern "C" int sa_output_norm_add(float* x, const void* y, int y_dtype, int parts, const float* w, const float* s,
+                                  void* h, int act_dtype, float eps, int T, int d, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (d <= 0 || parts < 1) return SA_ERR_ARG;
+  if (y && (!w || !s)) return SA_ERR_ARG;
+  if (y && y_dtype != act_dtype && y_dtype != SA_F32) return SA_ERR_UNSUPPORTED;
+  if (y && parts > 1 && y_dtype != SA_F32) return SA_ERR_UNSUPPORTED;
+  const size_t part_stride = (size_t)T * d;
+  dim3 grid(T), block(d >= 1024 ? 256 : (d >= 256 ? 128 : 64));
+#define GO(TA, TD)                                                                                          \
+  hipLaunchKernelGGL((output_norm_add_kernel<TA, TD>), grid, block, 0, stream, x, (const TD*)y, parts,      \
+                     part_stride, w, s, (TA*)h, eps, d)
+  const bool yfloat = !y || y_dtype == SA_F32;
+  if (act_dtype == SA_F32) GO(float, float);
+  else if (act_dtype == SA_BF16) { if (yfloat) GO(bf16_t, float); else GO(bf16_t, bf16_t); }
+  else return SA_ERR_UNSUPPORTED;
+#undef GO
+  SA_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// a[i] = act(a[i]) in place.  kind 0: gelu, tanh form: 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)));
+// kind 1: silu.
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float gelu_tanh_f(float z) {
+  const float u = 0.7978845608028654f * (z + 0.044715f * z * z * z);
+  return 0.5f * z * (1.f + tanhf(u));
+}
+
+template <typename TA>
+__global__ void activation_kernel(TA* __restrict__ a, size_t n, int kind) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    const float z = to_float(a[i]);
+    const float r = kind == 0 ? gelu_tanh_f(z) : z / (1.f + expf(-z));
+    a[i] = from_float<TA>(r);
+  }
+}
+
+extern "C" int sa_activation(void* a, int act_dtype, long long n, int kind, hipStream_t stream) {
+  if (n <= 0) return 0;
+  if (kind < 0 || kind > 1) return SA_ERR_ARG;
+  long long blocks = (n + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  dim3 grid((unsigned)blocks), block(256);
+  if (act_dtype == SA_F32) hipLaunchKernelGGL(activation_kernel<float>, grid, block, 0, stream, (float*)a, (size_t)n, kind);
+  else if (act_dtype == SA_BF16)
+    hipLaunchKernelGGL(activation_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)a, (size_t)n, kind);
+  else return SA_ERR_UNSUPPORTED;
+  SA_LAUNCH_CHECK();
+  return 0;
+}

@@ -75,6 +75,9 @@ class StepContext:
     prev_tokens: Optional[torch.Tensor] = None
     # where the head is asked to put the step's logits (fp32 [R, V]); None: wherever it likes
     logits_out: Optional[torch.Tensor] = None
+    # the residual stream in the activation dtype, where the layer that ran last has made that copy and
+    # the stream has not changed since (layers whose sublayers read the stream itself pass it on)
+    stream_copy: Optional[torch.Tensor] = None
 
 
 def _align(n: int) -> int:

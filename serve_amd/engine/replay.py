@@ -29,7 +29,7 @@ from .engine import Engine
 
 # granularity in which the trace's token budget is counted, per request
 TOKEN_ROUNDING = 64
-MAX_LIVE_REQUESTS = 16
+MAX_LIVE_REQUESTS = 4
 
 
 def replay_config(dtype: str, max_tokens: int, page_size: int = 16, device: str = "cuda:0") -> EngineConfig:

@@ -42,7 +42,8 @@ class Model:
         for i, ls in enumerate(spec.layers):
             arrangement = get_part("arrangement", ls.arrangement)
             roles = arrangement.PART_ROLES              # part name -> registry role
-            if set(ls.parts) != set(roles):
+            optional = set(getattr(arrangement, "OPTIONAL_PARTS", ()))      # (a layer without a feed-forward)
+            if not (set(roles) - optional) <= set(ls.parts) <= set(roles):
                 raise ValueError(f"layer {i}: arrangement {ls.arrangement!r} is built from the parts "
                                  f"{sorted(roles)}, the spec gives {sorted(ls.parts)}")
             self.layers.append(arrangement(**{name: _make(roles[name], ps) for name, ps in ls.parts.items()}))
@@ -164,6 +165,7 @@ class Model:
     def forward(self, ctx, caches: List[LayerCache]) -> torch.Tensor:
         """Run the tokens of one step; return fp32 logits [R, V] at ctx.logit_rows."""
         x = self.embedding.forward(ctx)
+        ctx.stream_copy = None          # (what a layer may leave for the next: the stream in the activation dtype)
         pending = None
         for e in self.spec.run_order:
             pending = self.layers[e.layer].forward(x, pending, ctx, caches[e.cache], e.writes_cache)

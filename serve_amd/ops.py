@@ -373,6 +373,229 @@ def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     return out
 
 
+# ---------------------------------------------------------------------------------------------
+# layers whose norm sits on the sublayer's output; plain activations
+# ---------------------------------------------------------------------------------------------
+
+def _f32vec(t: torch.Tensor, n: int, name: str) -> None:
+    _check(t.dtype == torch.float32 and t.numel() == n, f"{name} must be fp32 with {n} entries")
+
+
+def output_norm_add(x: torch.Tensor, y: Optional[torch.Tensor], weight: Optional[torch.Tensor],
+                    scale: Optional[torch.Tensor], eps: float, h: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    """x += (y / sqrt(mean(y^2) + eps) * weight) * scale on the fp32 residual stream x [T, d], in place;
+    `h` (activation dtype [T, d]) receives a copy of the new x.  y is [T, d] in h's dtype or fp32, or
+    fp32 [parts, T, d] partial sums that are added in order.  y None: only the copy is made."""
+    _dev(x, y, weight, scale, h)
+    _check(x.dtype == torch.float32 and x.dim() == 2, "residual stream must be fp32 [T, d]")
+    T, d = x.shape
+    act = h.dtype if h is not None else (y.dtype if y is not None and y.dim() == 2 else torch.float32)
+    parts, ycode = 1, F32
+    if y is not None:
+        _f32vec(weight, d, "norm weight")
+        _f32vec(scale, d, "layer scale")
+        if y.dim() == 3:
+            parts = y.shape[0]
+            _check(y.dtype == torch.float32 and y.shape[1:] == (T, d), "partial sums must be fp32 [parts, T, d]")
+        else:
+            _check(y.shape == (T, d) and y.dtype in (act, torch.float32), "y must be [T, d] in the activation dtype or fp32")
+        ycode = _code(y)
+    if h is not None:
+        _check(h.shape == (T, d), "the stream's copy must be [T, d]")
+    lib = load_library("sublayer")
+    _ret(lib.sa_output_norm_add(_ptr(x), _ptr(y), c_int(ycode), c_int(parts), _ptr(weight), _ptr(scale), _ptr(h),
+                                c_int(_DT[act]), c_float(eps), c_int(T), c_int(d), _stream()), "output_norm_add")
+    return h
+
+
+ACTIVATIONS = {"gelu_tanh": 0, "silu": 1}
+
+
+def activation(a: torch.Tensor, kind: str) -> torch.Tensor:
+    """a = act(a) in place: 'gelu_tanh' (0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))) or 'silu'."""
+    _dev(a)
+    _check(kind in ACTIVATIONS, f"unknown activation {kind!r}; known: {sorted(ACTIVATIONS)}")
+    lib = load_library("sublayer")
+    _ret(lib.sa_activation(_ptr(a), c_int(_code(a)), ctypes.c_longlong(a.numel()), c_int(ACTIVATIONS[kind]),
+                           _stream()), "activation")
+    return a
+
+
+# ---------------------------------------------------------------------------------------------
+# gated delta rule
+# ---------------------------------------------------------------------------------------------
+DELTA_MAX_DIM = 256
+DELTA_MAX_TAPS = 16
+
+
+def delta_rule(z: torch.Tensor, conv_w: torch.Tensor, ba: torch.Tensor, A_log: torch.Tensor, dt_bias: torch.Tensor,
+               norm_w: torch.Tensor, state: torch.Tensor, ctx, y: torch.Tensor, eps: float, heads: int,
+               kv_heads: int, dk: int, dv: int, taps: int) -> torch.Tensor:
+    """The gated delta rule over the step's tokens.  z [T, >= C + H dv]: the projections
+    [q: Hk dk | k: Hk dk | v: H dv | gate: H dv] (C = the first three: the convolution's channels);
+    conv_w fp32 [C, taps]; ba fp32 [T, 2 H] (beta's logits, then the decay's); state fp32
+    [slots, H dk dv + (taps - 1) C], a request's row (ctx.state_slots, -1: none) read and written;
+    y [T, H dv] in z's dtype: the normed, gated read-out."""
+    _dev(z, conv_w, ba, A_log, dt_bias, norm_w, state, y, ctx.seg_of_token, ctx.cu_q, ctx.state_slots)
+    T, B = ctx.num_tokens, ctx.num_segments
+    H, Hk = heads, kv_heads
+    C = 2 * Hk * dk + H * dv
+    _check(z.dim() == 2 and z.shape[0] == T and z.shape[1] >= C + H * dv, f"z must be [T, >= {C + H * dv}]")
+    _check(H % Hk == 0 and 0 < dk <= DELTA_MAX_DIM and 0 < dv <= DELTA_MAX_DIM and 1 <= taps <= DELTA_MAX_TAPS,
+           f"delta rule: head sizes up to {DELTA_MAX_DIM}, up to {DELTA_MAX_TAPS} taps")
+    _check(conv_w.dtype == torch.float32 and conv_w.shape == (C, taps), f"conv_w must be fp32 [{C}, {taps}]")
+    _check(ba.dtype == torch.float32 and ba.shape == (T, 2 * H), f"ba must be fp32 [T, {2 * H}]")
+    _f32vec(A_log, H, "A_log")
+    _f32vec(dt_bias, H, "dt_bias")
+    _f32vec(norm_w, dv, "norm weight")
+    need = H * dk * dv + (taps - 1) * C
+    _check(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] >= need,
+           f"state rows must be fp32 with at least {need} entries")
+    _check(y.shape == (T, H * dv) and y.dtype == z.dtype, "y must be [T, H dv] in z's dtype")
+    _i32(ctx.seg_of_token, T, "seg_of_token")
+    _i32(ctx.cu_q, B + 1, "cu_q")
+    _i32(ctx.state_slots, B, "state_slots")
+    lib = load_library("delta_rule")
+    lib.sa_delta_rule_work_floats.restype = ctypes.c_longlong
+    work = torch.empty(int(lib.sa_delta_rule_work_floats(c_int(T), c_int(H), c_int(Hk), c_int(dk), c_int(dv))),
+                       dtype=torch.float32, device=z.device)
+    _ret(lib.sa_delta_rule(_ptr(z), c_int(_code(z)), c_int(z.shape[1]), _ptr(conv_w), _ptr(ba), _ptr(A_log),
+                           _ptr(dt_bias), _ptr(norm_w), _ptr(state), ctypes.c_longlong(state.shape[1]),
+                           _ptr(ctx.seg_of_token), _ptr(ctx.cu_q), _ptr(ctx.state_slots), _ptr(work), _ptr(y),
+                           c_float(eps), c_int(T), c_int(B), c_int(H), c_int(Hk), c_int(dk), c_int(dv), c_int(taps),
+                           _stream()), "delta_rule")
+    return y
+
+
+# ---------------------------------------------------------------------------------------------
+# latent attention
+# ---------------------------------------------------------------------------------------------
+
+def latent_kv_write(z: torch.Tensor, norm_w: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor,
+                    slots: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, eps: float, rank: int,
+                    rot_dim: int) -> None:
+    """z [T, rank + rot_dim] -> the token's cache rows: k_pages [P, 1, page, Dp] gets
+    [normed latent | rotated key part | 0], v_pages [P, 1, Dp, page] the normed latent (and zeros)."""
+    _dev(z, norm_w, positions, inv_freq, slots, k_pages, v_pages)
+    T = z.shape[0]
+    _check(z.dim() == 2 and z.shape[1] == rank + rot_dim, f"z must be [T, {rank + rot_dim}]")
+    P, one, page_size, Dp = k_pages.shape
+    _check(one == 1 and Dp >= rank + rot_dim and v_pages.shape == (P, 1, Dp, page_size),
+           "latent pages must be [P, 1, page, Dp] and [P, 1, Dp, page]")
+    _check(k_pages.dtype == z.dtype and v_pages.dtype == z.dtype, "cache dtype must match activations")
+    _f32vec(norm_w, rank, "latent norm weight")
+    _f32vec(inv_freq, rot_dim // 2, "inv_freq")
+    _i32(positions, T, "positions")
+    _i32(slots, T, "slots")
+    lib = load_library("latent")
+    _ret(lib.sa_latent_kv_write(_ptr(z), c_int(_code(z)), _ptr(norm_w), _ptr(positions), _ptr(inv_freq), _ptr(slots),
+                                _ptr(k_pages), _ptr(v_pages), c_float(eps), c_int(T), c_int(rank), c_int(rot_dim),
+                                c_int(Dp), c_int(page_size), _stream()), "latent_kv_write")
+
+
+def head_linear(x: torch.Tensor, in_stride: int, in_head_stride: int, w: torch.Tensor, out: torch.Tensor,
+                out_stride: int, out_head_stride: int, T: int) -> torch.Tensor:
+    """out[t, h, :N] = x[t, h, :K] @ w[h] for w [H, K, N]: head h's K inputs of token t start at element
+    t * in_stride + h * in_head_stride of x, its N outputs at t * out_stride + h * out_head_stride of out."""
+    _dev(x, w, out)
+    _check(w.dim() == 3 and x.dtype == w.dtype == out.dtype, "head_linear: w must be [H, K, N], one dtype throughout")
+    H, K, N = w.shape
+    if T:
+        _check(x.numel() >= (T - 1) * in_stride + (H - 1) * in_head_stride + K, "head_linear: input too short")
+        _check(out.numel() >= (T - 1) * out_stride + (H - 1) * out_head_stride + N, "head_linear: output too short")
+    lib = load_library("latent")
+    _ret(lib.sa_head_linear(_ptr(x), c_int(in_stride), c_int(in_head_stride), _ptr(w), _ptr(out), c_int(out_stride),
+                            c_int(out_head_stride), c_int(_code(x)), c_int(T), c_int(H), c_int(K), c_int(N), _stream()),
+         "head_linear")
+    return out
+
+
+def latent_q_rot(q: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor, qf: torch.Tensor, heads: int,
+                 dim: int, rot_dim: int, rank: int) -> None:
+    """The rotated part of every query head into its place behind the `rank` latent dims of the head's
+    row of qf [T, H Dp], and zeros behind it.  q [T, H (dim + rot_dim)]."""
+    _dev(q, positions, inv_freq, qf)
+    T = q.shape[0]
+    _check(q.shape == (T, heads * (dim + rot_dim)) and qf.dim() == 2 and qf.shape[0] == T and qf.shape[1] % heads == 0
+           and qf.dtype == q.dtype, "latent_q_rot: q [T, H (dim + rot_dim)], qf [T, H Dp]")
+    Dp = qf.shape[1] // heads
+    _check(Dp >= rank + rot_dim, "latent_q_rot: rows of qf are too short")
+    _f32vec(inv_freq, rot_dim // 2, "inv_freq")
+    _i32(positions, T, "positions")
+    lib = load_library("latent")
+    _ret(lib.sa_latent_q_rot(_ptr(q), c_int(_code(q)), _ptr(positions), _ptr(inv_freq), _ptr(qf), c_int(T),
+                             c_int(heads), c_int(dim), c_int(rot_dim), c_int(rank), c_int(Dp), _stream()), "latent_q_rot")
+
+
+# ---------------------------------------------------------------------------------------------
+# routed experts
+# ---------------------------------------------------------------------------------------------
+
+def moe_route(logits: torch.Tensor, experts: int, top: int, ids: torch.Tensor, weights: torch.Tensor) -> None:
+    """Per row of logits fp32 [T, >= experts]: the `top` experts with the largest logits (ids int32
+    [T, top]) and the softmax over those logits alone (weights fp32 [T, top])."""
+    _dev(logits, ids, weights)
+    T = logits.shape[0]
+    _check(logits.dtype == torch.float32 and logits.dim() == 2 and logits.shape[1] >= experts, "router logits must be fp32 [T, >= E]")
+    _check(0 < top <= experts, "top must be within the number of experts")
+    _check(ids.dtype == torch.int32 and ids.shape == (T, top) and weights.dtype == torch.float32 and weights.shape == (T, top),
+           "ids int32 [T, top], weights fp32 [T, top]")
+    lib = load_library("moe")
+    _ret(lib.sa_moe_route(_ptr(logits), c_int(logits.shape[1]), _ptr(ids), _ptr(weights), c_int(T), c_int(experts),
+                          c_int(top), _stream()), "moe_route")
+
+
+def moe_experts(h: torch.Tensor, ids: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor,
+                yk: torch.Tensor) -> torch.Tensor:
+    """yk[t * top + k] = expert ids[t, k] applied to h[t]: down(silu(gate h) * up h), fp32 [T top, d].
+    w_gate, w_up [E, F, d], w_down [E, d, F] in h's dtype."""
+    _dev(h, ids, w_gate, w_up, w_down, yk)
+    T, d = h.shape
+    top = ids.shape[1]
+    E, F, d2 = w_gate.shape
+    _check(d2 == d and w_up.shape == (E, F, d) and w_down.shape == (E, d, F), "expert matrices must be [E, F, d], [E, F, d], [E, d, F]")
+    _check(w_gate.dtype == h.dtype and w_up.dtype == h.dtype and w_down.dtype == h.dtype, "experts and activations must share a dtype")
+    _check(ids.dtype == torch.int32 and ids.shape == (T, top), "ids must be int32 [T, top]")
+    _check(yk.dtype == torch.float32 and yk.shape == (T * top, d), "yk must be fp32 [T top, d]")
+    lib = load_library("moe")
+    n = T * top
+    tiles = int(lib.sa_moe_max_tiles(c_int(n), c_int(E)))
+    ints = torch.empty(2 * E + 1 + n + 2 * tiles + 1, dtype=torch.int32, device=h.device)
+    act = torch.empty((n, F), dtype=h.dtype, device=h.device)
+    _ret(lib.sa_moe_experts(_ptr(h), c_int(_code(h)), _ptr(ids), _ptr(w_gate), _ptr(w_up), _ptr(w_down), _ptr(ints),
+                            _ptr(act), _ptr(yk), c_int(T), c_int(top), c_int(E), c_int(d), c_int(F), _stream()),
+         "moe_experts")
+    return yk
+
+
+def moe_combine(yk: torch.Tensor, weights: torch.Tensor, shared: Optional[torch.Tensor],
+                logits: Optional[torch.Tensor], gate_col: int, y: torch.Tensor) -> torch.Tensor:
+    """y[t] = sum_k weights[t, k] yk[t top + k] (+ sigmoid(logits[t, gate_col]) * shared[t]);
+    shared [T, d] or fp32 [parts, T, d]; logits None: the shared rows are added as they are."""
+    _dev(yk, weights, shared, logits, y)
+    T, top = weights.shape
+    d = y.shape[1]
+    _check(y.dtype == torch.float32 and y.shape == (T, d) and yk.shape == (T * top, d) and yk.dtype == torch.float32
+           and weights.dtype == torch.float32, "moe_combine: fp32 y [T, d], yk [T top, d], weights [T, top]")
+    parts, scode = 1, F32
+    if shared is not None:
+        if shared.dim() == 3:
+            parts = shared.shape[0]
+            _check(shared.dtype == torch.float32 and shared.shape[1:] == (T, d), "shared partial sums must be fp32 [parts, T, d]")
+        else:
+            _check(shared.shape == (T, d), "shared rows must be [T, d]")
+        scode = _code(shared)
+    gate, ldz = c_void_p(0), 0
+    if logits is not None:
+        _check(logits.dtype == torch.float32 and logits.dim() == 2 and logits.shape[0] == T
+               and 0 <= gate_col < logits.shape[1], "gate logits must be a column of fp32 [T, n]")
+        gate, ldz = c_void_p(logits.data_ptr() + 4 * gate_col), logits.shape[1]
+    lib = load_library("moe")
+    _ret(lib.sa_moe_combine(_ptr(yk), _ptr(weights), _ptr(shared), c_int(scode), c_int(parts), gate,
+                            c_int(ldz), _ptr(y), c_int(T), c_int(top), c_int(d), _stream()), "moe_combine")
+    return y
+
+
 _SINKS = {}
 
 

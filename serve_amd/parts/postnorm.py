@@ -1,0 +1,98 @@
+"""Layers whose norm sits on the sublayer's output:
+
+    x <- x + s1 * N1(mixer(x));   x <- x + s2 * N2(ffn(x))     N(y) = y / sqrt(mean(y^2) + eps) * (offset + w)
+
+The sublayers read the residual stream itself (its copy in the activation dtype), the norm
+weights may be stored around zero (`offset` 1), and every sublayer's normed output is scaled
+element by element (`scale`, a "layer scale") before it joins the stream.  A layer may have no
+feed-forward.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from .. import ops
+from ..registry import register_part
+from .base import LayerCache, ParamRequest, Part, Runtime
+
+
+class ScaledOutputNorm(Part):
+    """x += scale * (y / sqrt(mean(y^2) + eps) * (offset + weight)) on the fp32 stream, in one kernel
+    that also hands back the new stream in the activation dtype for the sublayer that reads it next."""
+
+    graph_safe = True
+
+    def __init__(self, size: int, eps: float, offset: float = 0.0):
+        self.size, self.eps, self.offset = int(size), float(eps), float(offset)
+
+    def param_requests(self) -> List[ParamRequest]:
+        return [ParamRequest("weight", (self.size,), init="normal:0.2" if self.offset else "ones_normal"),
+                ParamRequest("scale", (self.size,), init="ones_normal:0.2")]
+
+    def load(self, tensors, rt: Runtime) -> None:
+        self.rt = rt
+        self.weight = (tensors["weight"].float() + self.offset).contiguous()       # fp32, whatever the storage
+        self.scale = tensors["scale"].float().contiguous()
+
+    def forward(self, x: torch.Tensor, y: Optional[torch.Tensor], rows=None) -> torch.Tensor:
+        """Add the normed, scaled `y` into x (in place) and return what the next sublayer reads: x
+        itself in the float32 engine, else its copy in the activation dtype."""
+        if rows is not None:
+            raise ValueError("a norm on a sublayer's output takes whole steps, not rows")
+        h = None if self.rt.exact else self.rt.empty(tuple(x.shape))
+        ops.output_norm_add(x, y, self.weight, self.scale, self.eps, h)
+        return x if h is None else h
+
+
+def stream_copy(x: torch.Tensor, rt: Runtime) -> torch.Tensor:
+    """The fp32 stream as the sublayers read it."""
+    if rt.exact:
+        return x
+    return ops.output_norm_add(x, None, None, None, 0.0, rt.empty(tuple(x.shape)))
+
+
+class PostNormResidual:
+    """x += s1 N1(mixer(x)); x += s2 N2(ffn(x)), the second half only if the layer has a feed-forward.
+
+    It leaves no pending output: the stream is complete when the layer returns.  The copy of the
+    stream in the activation dtype that its last norm made travels to the next layer of this kind
+    on the step's context, so that only the first such layer of a model makes one itself."""
+
+    PART_ROLES = {"mixer": "mixer", "ffn": "feed_forward", "mixer_norm": "norm", "ffn_norm": "norm"}
+    OPTIONAL_PARTS = ("ffn", "ffn_norm")
+
+    def __init__(self, mixer, mixer_norm, ffn=None, ffn_norm=None):
+        if (ffn is None) != (ffn_norm is None):
+            raise ValueError("a feed-forward and its norm come together")
+        self.mixer, self.ffn, self.mixer_norm, self.ffn_norm = mixer, ffn, mixer_norm, ffn_norm
+
+    def cache_owner(self) -> Part:
+        return self.mixer
+
+    def parts(self) -> Dict[str, Part]:
+        out = {"mixer": self.mixer, "mixer_norm": self.mixer_norm}
+        if self.ffn is not None:
+            out.update(ffn=self.ffn, ffn_norm=self.ffn_norm)
+        return out
+
+    def forward(self, x: torch.Tensor, pending: Optional[torch.Tensor], ctx, cache: LayerCache,
+                writes_cache: bool = True) -> None:
+        rt = self.mixer_norm.rt
+        kept = getattr(ctx, "stream_copy", None)
+        ctx.stream_copy = None
+        if pending is not None:
+            # a layer of another arrangement left its last output unadded
+            x.add_(pending.sum(0) if pending.dim() == 3 else pending)
+            kept = None
+        h = kept if kept is not None else stream_copy(x, rt)
+        h = self.mixer_norm.forward(x, self.mixer.forward(h, ctx, cache, writes_cache))
+        if self.ffn is not None:
+            h = self.ffn_norm.forward(x, self.ffn.forward(h, ctx))
+        ctx.stream_copy = h
+        return None
+
+
+register_part("norm", "scaled_output_rmsnorm", ScaledOutputNorm)
+register_part("arrangement", "postnorm_residual", PostNormResidual)

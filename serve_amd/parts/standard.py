@@ -33,15 +33,19 @@ class RMSNorm(Part):
 
     graph_safe = True
 
-    def __init__(self, size: int, eps: float):
-        self.size, self.eps = int(size), float(eps)
+    def __init__(self, size: int, eps: float, offset: float = 0.0):
+        """`offset`: what is added to the stored weight before it multiplies (1.0 for checkpoints
+        that keep their norm weights around zero); the sum is made in fp32 when the part loads."""
+        self.size, self.eps, self.offset = int(size), float(eps), float(offset)
 
     def param_requests(self) -> List[ParamRequest]:
-        return [ParamRequest("weight", (self.size,), init="ones_normal")]
+        return [ParamRequest("weight", (self.size,), init="normal:0.2" if self.offset else "ones_normal")]
 
     def load(self, tensors, rt: Runtime) -> None:
         self.rt = rt
         self.weight = tensors["weight"]
+        if self.offset:
+            self.weight = self.weight.float() + self.offset
 
     def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor],
                 rows: Optional[torch.Tensor] = None) -> torch.Tensor:

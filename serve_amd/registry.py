@@ -65,6 +65,8 @@ def load_config(folder: str):
     with open(path) as f:
         raw = json.load(f)
     names = raw.get("architectures")
+    if not names and isinstance(raw.get("architecture"), str):
+        names = [raw["architecture"]]           # (files that name their one architecture as a string)
     if not names:
         raise KeyError(f"{path} has no 'architectures' entry; known architectures: {known_architectures()}")
     arch = get_architecture(names[0])
@@ -80,3 +82,4 @@ def _ensure_builtin() -> None:
         _builtin_loaded = True
         from . import parts  # noqa: F401  (registers the part kinds)
         from .models import llama  # noqa: F401  (registers LlamaForCausalLM)
+        from .models import zozosun  # noqa: F401  (registers Zozosun)

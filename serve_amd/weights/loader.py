@@ -100,8 +100,9 @@ def _tensor_seed(seed: int, name: str) -> int:
 
 def random_tensors(model: Model, seed: int, dtype: torch.dtype = torch.bfloat16,
                    scales: Optional[Dict[str, float]] = None) -> Iterator[Tuple[str, torch.Tensor]]:
-    """One tensor per request, a pure function of (seed, tensor name): matrices N(0, 0.02), norm
-    weights 1 + N(0, 0.1), drawn in fp32 on the CPU and rounded to `dtype`.  A tensor that only
+    """One tensor per request, a pure function of (seed, tensor name): by the request's `init` rule,
+    matrices N(0, 0.02) ("normal"), norm weights 1 + N(0, 0.1) ("ones_normal"), or with the deviation
+    the rule names ("normal:0.2"), or uniform ("uniform:-3:0"); drawn in fp32 on the CPU and rounded to `dtype`.  A tensor that only
     stands for another part's (a tied output matrix) is not produced.  `scales` maps a regular
     expression to a factor for the matrices whose checkpoint name it matches (a model whose
     attention scores are of order one instead of 0.03 needs larger q and k projections)."""
@@ -112,13 +113,21 @@ def random_tensors(model: Model, seed: int, dtype: torch.dtype = torch.bfloat16,
         g = torch.Generator(device="cpu")
         g.manual_seed(_tensor_seed(seed, r.checkpoint_name))
         t = torch.randn(r.shape, generator=g, dtype=torch.float32)
-        if r.init == "ones_normal":
-            t = 1.0 + 0.1 * t
-        elif r.init == "normal":
-            t = 0.02 * t
+        kind, _, args = r.init.partition(":")
+        try:
+            nums = [float(a) for a in args.split(":")] if args else []
+        except ValueError:
+            raise ValueError(f"unknown init rule {r.init!r} for {r.checkpoint_name}") from None
+        if kind == "ones_normal" and len(nums) <= 1:          # 1 + N(0, std), std 0.1 unless given
+            t = 1.0 + (nums[0] if nums else 0.1) * t
+        elif kind == "normal" and len(nums) <= 1:             # N(0, std), std 0.02 unless given
+            t = (nums[0] if nums else 0.02) * t
             for pattern, factor in rules:
                 if pattern.search(r.checkpoint_name):
                     t = t * factor
+        elif kind == "uniform" and len(nums) == 2:            # U(lo, hi)
+            u = torch.rand(r.shape, generator=g, dtype=torch.float32)
+            t = nums[0] + (nums[1] - nums[0]) * u
         else:
             raise ValueError(f"unknown init rule {r.init!r} for {r.checkpoint_name}")
         yield r.checkpoint_name, t.to(dtype)

@@ -221,6 +221,45 @@ def report(engine, cfg, steps: int, warmup: int, make_engine=None) -> int:
     return 0
 
 
+def designs(args) -> int:
+    """`--designs`: prefill and decode throughput of the Zozosun shapes, each beside the Llama shape of the same
+    width, depth, vocabulary and feed-forward width (serve_amd.benchmark.DESIGN_PAIRS), random weights.  One
+    JSON line per model: tokens/s of a 2,048-token prompt, and of decode steps at batch 1, 8 and 64 with
+    contexts around `--context`; with the bytes a decode step streams and the flops of the prompt as the
+    models' parts account for them."""
+    import torch
+    from serve_amd.benchmark import DESIGN_PAIRS, SHAPES
+    from serve_amd.config.engine import EngineConfig
+    from serve_amd.engine.engine import Engine
+    page, context = 16, min(args.context, 2048)
+    names = [n for pair in DESIGN_PAIRS for n in pair if args.shape in ("llama-1b", n, pair[0])]
+    for name in names:
+        ecfg = EngineConfig(dtype=args.dtype, page_size=page, num_pages=64 * (-(-context // page)) + 512,
+                            max_context=max(context, 2048), max_requests=64, max_tokens_per_step=2048 + 64,
+                            prefill_chunk=2048, admission="reserve")
+        engine = Engine.from_config(SHAPES[name], seed=0, cfg=ecfg,
+                                    weight_dtype=torch.bfloat16 if args.dtype == "bfloat16" else torch.float32)
+        item = ITEM[args.dtype]
+        out = {"model": name, "dtype": args.dtype, "layers": len(engine.model.spec.run_order),
+               "weights_read_by_a_decode_step_GB": round(weight_bytes(engine.model, item) / 1e9, 3)}
+        T = 2048
+        pt = prefill_run(engine, T, repeats=3, seed=7)
+        fl = prefill_flops(engine.model, T)
+        out["prefill"] = {"tokens": T, "ms": round(pt * 1e3, 3), "tokens_per_s": round(T / pt, 1),
+                          "TFLOP": round(fl / 1e12, 3), "PFLOP_per_s": round(fl / pt / 1e15, 4)}
+        for b in (1, 8, 64):
+            steps = args.steps
+            prompt_len = context - steps - 8 - 3 - head_start(engine, b, context)
+            dt, mean_ctx = decode_run(engine, b, prompt_len, 8, steps, seed=10 + b)
+            nbytes = weight_bytes(engine.model, item) + b * kv_bytes(engine.model, mean_ctx, item)
+            out[f"decode_b{b}"] = {"ms_per_step": round(dt / steps * 1e3, 4), "tokens_per_s": round(b * steps / dt, 1),
+                                   "context": int(mean_ctx), "TB_per_s": round(nbytes / (dt / steps) / 1e12, 3)}
+        print(json.dumps(out), flush=True)
+        del engine
+        torch.cuda.empty_cache()
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -243,6 +282,9 @@ def main() -> int:
     ap.add_argument("--report", action="store_true",
                     help="print a table instead of the JSON line: decode at batch 1, 8 and 64 and the prefill, each "
                     "with its bytes or flops, as a share of the published peaks and of ceilings measured here")
+    ap.add_argument("--designs", action="store_true",
+                    help="measure the Zozosun shapes beside Llama shapes of equal size instead (prefill of 2,048 tokens, "
+                    "decode at batch 1, 8 and 64); one JSON line per model; --shape picks one pair")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -252,6 +294,8 @@ def main() -> int:
     from serve_amd.config.engine import EngineConfig
     from serve_amd.engine.engine import Engine
 
+    if args.designs:
+        return designs(args)
     cfg = model_config(args.layers, args.shape)
     full_layers = model_config(0, args.shape).num_hidden_layers
     shape_name = {"llama-1b": "Llama-3.2-1B", "llama-3b": "Llama-3.2-3B", "llama-8b": "Llama-3.1-8B"}.get(args.shape, args.shape)

@@ -48,6 +48,40 @@ SHAPES = {
 }
 
 
+def _zozosun_shape(width: int, vocab: int, groups: int, delta_heads: int, attn_heads: int, ff: int, experts: int,
+                   top: int, expert_ff: int, shared_ff: int, window: int):
+    """A Zozosun shape at the sizes of a real model's layers: `groups` times four layers, delta rule + dense,
+    delta rule + experts, latent attention + dense, latent attention on the cache of the layer before + experts.
+    The latent row (kv_rank 96 + 32 rotated dims) is as wide as the matrix-core attention's widest head."""
+    from .config.zozosun import (DeltaMixerConfig, DenseMlpConfig, LatentMixerConfig, MoeMlpConfig, ZozosunConfig,
+                                 ZozosunLayerConfig)
+    delta = DeltaMixerConfig(heads=delta_heads, kv_heads=delta_heads // 2, dim=128, vdim=128, conv=4)
+    layers = []
+    for g in range(groups):
+        latent = LatentMixerConfig(heads=attn_heads, dim=64, rot_dim=32, vdim=64, kv_rank=96, scale=96 ** -0.5,
+                                   rot_base=1.0e6, window=window)
+        reader = LatentMixerConfig(heads=attn_heads, dim=64, rot_dim=32, vdim=64, kv_rank=96, scale=96 ** -0.5,
+                                   rot_base=1.0e6, window=window, kv_from=4 * g + 2)
+        moe = MoeMlpConfig(experts, top, expert_ff, shared_ff)
+        layers += [ZozosunLayerConfig(delta, DenseMlpConfig(ff)), ZozosunLayerConfig(delta, moe),
+                   ZozosunLayerConfig(latent, DenseMlpConfig(ff)), ZozosunLayerConfig(reader, moe)]
+    return ZozosunConfig(vocab=vocab, width=width, eps=1e-5, layers=tuple(layers))
+
+
+# Zozosun at two widths, and beside each a Llama shape of the same width, depth, vocabulary and feed-forward
+# width (the closest model the engine has): `bench.py --designs` measures them side by side
+SHAPES.update({
+    "zozosun-tiny": _zozosun_shape(64, 512, 1, 2, 2, 128, 4, 2, 32, 64, 24),
+    "zozosun-2k": _zozosun_shape(2048, 32768, 2, 16, 16, 8192, 32, 4, 1024, 2048, 1024),
+    "zozosun-4k": _zozosun_shape(4096, 32768, 1, 32, 32, 14336, 64, 6, 1536, 3072, 1024),
+    "llama-2k": LlamaConfig(vocab_size=32768, hidden_size=2048, intermediate_size=8192, num_hidden_layers=8,
+                            num_attention_heads=32, num_key_value_heads=8, head_dim=64, rope_theta=500000.0),
+    "llama-4k": LlamaConfig(vocab_size=32768, hidden_size=4096, intermediate_size=14336, num_hidden_layers=4,
+                            num_attention_heads=32, num_key_value_heads=8, head_dim=128, rope_theta=500000.0),
+})
+DESIGN_PAIRS = (("zozosun-2k", "llama-2k"), ("zozosun-4k", "llama-4k"))
+
+
 def generate_requests(input_length: int, output_length: int, num_sequences: int, vocab_size: int,
                       fixed_lengths: bool = False, seed: int = 1352, min_input_length: int = 1,
                       fixed_output_length: bool = False):

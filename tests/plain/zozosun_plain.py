@@ -141,7 +141,9 @@ def latent_attention(h: Tensor, W: Dict[str, Tensor], p: str, m: dict, c: Tensor
     scores = (torch.einsum("ihd,jhd->hij", qn, kn) + torch.einsum("ihd,jd->hij", qr, kr)) * m["scale"]
     i = torch.arange(T)[:, None]
     j = torch.arange(T)[None, :]
-    seen = (i - j >= 0) & (i - j < m["mask"]["size"])
+    seen = i - j >= 0
+    if m.get("mask"):                                  # a sliding window: itself and the size - 1 tokens before it
+        seen = seen & (i - j < m["mask"]["size"])
     scores = scores.masked_fill(~seen, float("-inf"))
     out = torch.einsum("hij,jhd->ihd", torch.softmax(scores, dim=-1), val)
     return out.reshape(T, H * dv) @ W[p + "o"].t()
@@ -158,7 +160,7 @@ def gated_expert(h: Tensor, W: Dict[str, Tensor], p: str) -> Tensor:
     return (silu(h @ W[p + "gate"].t()) * (h @ W[p + "up"].t())) @ W[p + "down"].t()
 
 
-def moe_ff(h: Tensor, W: Dict[str, Tensor], p: str, mlp: dict) -> Tensor:
+def moe_ff(h: Tensor, W: Dict[str, Tensor], p: str, mlp: dict, margins: Optional[list] = None) -> Tensor:
     """Every token takes its `top` experts with the largest router logits, weighted by the softmax
     over those logits alone; a shared expert, if there is one, is added for every token, times
     sigmoid(W_sg h)."""
@@ -166,7 +168,11 @@ def moe_ff(h: Tensor, W: Dict[str, Tensor], p: str, mlp: dict) -> Tensor:
     z = h @ W[p + "router"].t()                                     # [T, E]
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
-        chosen = sorted(range(E), key=lambda e: -float(z[t, e]))[:top]
+        order = sorted(range(E), key=lambda e: -float(z[t, e]))
+        chosen = order[:top]
+        if margins is not None and top < E:
+            # by how much the last chosen logit leads the first that is left out, in units of the logits' spread
+            margins.append((t, float((z[t, order[top - 1]] - z[t, order[top]]) / z[t].std().clamp_min(1e-12))))
         w = torch.softmax(z[t, chosen], dim=0)
         for wi, e in zip(w, chosen):
             out[t] += wi * gated_expert(h[t:t + 1], W, f"{p}e{e}.")[0]
@@ -179,8 +185,9 @@ def moe_ff(h: Tensor, W: Dict[str, Tensor], p: str, mlp: dict) -> Tensor:
 # the model
 # --------------------------------------------------------------------------------------
 def forward(tokens: Sequence[int], weights: Dict[str, Tensor], cfg: dict, dtype=torch.float64,
-            return_layers: bool = False):
-    """Logits [T, vocab] of one sequence (and, on request, the residual stream after every layer)."""
+            return_layers: bool = False, margins: Optional[list] = None):
+    """Logits [T, vocab] of one sequence (and, on request, the residual stream after every layer).
+    `margins` receives (token, margin) of every routing decision: how clearly the experts were chosen."""
     W = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in weights.items()}
     eps = cfg["norm"]["eps"]
     x = W["embed"][torch.as_tensor(list(tokens), dtype=torch.long)]
@@ -201,7 +208,7 @@ def forward(tokens: Sequence[int], weights: Dict[str, Tensor], cfg: dict, dtype=
         x = x + norm_around_zero(y, W[p + "norm1"], eps) * W[p + "ls1"]
         mlp = layer.get("mlp")
         if mlp is not None:
-            y = dense_ff(x, W, p + "mlp.") if mlp["kind"] == "dense" else moe_ff(x, W, p + "mlp.", mlp)
+            y = dense_ff(x, W, p + "mlp.") if mlp["kind"] == "dense" else moe_ff(x, W, p + "mlp.", mlp, margins)
             x = x + norm_around_zero(y, W[p + "norm2"], eps) * W[p + "ls2"]
         streams.append(x)
     logits = norm_around_zero(x, W["final.norm"], eps) @ W["head"].t()

@@ -120,8 +120,12 @@ def test_unequal_requests_together_with_pages_and_slots_used_again(tmp_path, nam
             engine.runner.release(k)
         engine.runner.cache.check_invariants()
     assert any(len(v) > 1 for v in slots_seen.values()), "no state slot was used twice"
-    for k, toks in reqs.items():
-        zm.assert_matches_plain(torch.cat(rows[k]), folder, toks, dtype, f"{name} request {k} in the mix")
+    pairs = [zm.kept_rows(torch.cat(rows[k]), folder, toks, dtype, f"{name} request {k} in the mix") for k, toks in reqs.items()]
+    if dtype == "float32":
+        for (got, want), k in zip(pairs, reqs):
+            zm.assert_rows_close(got, want, dtype, f"{name} request {k} in the mix")
+    zm.assert_close_but_few(torch.cat([g.cpu() for g, _ in pairs]), torch.cat([w for _, w in pairs]), dtype,
+                            f"{name}: all requests of the mix")
 
 
 def _with_windows(config: dict, shift: int) -> dict:

@@ -115,27 +115,29 @@ __global__ __launch_bounds__(256) void delta_conv_state_kernel(
 }
 
 // ---------------------------------------------------------------------------------------------
-// (3) the recurrence.  grid (ceil(dv / COLS), H, B); a wave holds 16 columns of S, each cut in four
-// parts along dk (a thread keeps RPT rows of one column in registers), so that S^T k and S^T q are
-// sums inside a thread plus two exchanges between neighbouring lanes.  The tokens of a segment come
-// through LDS in chunks of CH; a segment's state is read once and written once.
+// (3) the recurrence.  grid (ceil(dv / cols), H, B).  A column of S is cut in R parts along dk: a thread
+// keeps RPT rows of one column in registers, so that S^T k and S^T q are sums inside a thread plus
+// log2(R) exchanges between neighbouring lanes.  R = 4 (a wave holds 16 columns) for steps of single
+// tokens, where reading and writing the state is the work and neighbouring lanes should touch
+// neighbouring columns; R = 16 (a wave holds 4 columns, a head is spread over four times as many waves)
+// for prompt portions, where the tokens of a segment form one chain of dependent steps and the length of
+// a step is what counts.  The tokens of a segment come through LDS in chunks of CH; a segment's state is
+// read once and written once.
 // ---------------------------------------------------------------------------------------------
-#define DR_CH 16
-
-template <int RPT>
+template <int RPT, int R, int CH>
 __global__ __launch_bounds__(256) void delta_recurrence_kernel(
     const float* __restrict__ qn, const float* __restrict__ kn, const float* __restrict__ vc,
     const float* __restrict__ beta, const float* __restrict__ decay, float* __restrict__ state,
     size_t state_stride, const int* __restrict__ cu_q, const int* __restrict__ state_slots,
     float* __restrict__ o, int H, int Hk, int dk, int dv) {
-  constexpr int PAD = RPT + 4;           // a part's rows in LDS, padded so that the four parts lie in other banks
-  constexpr int ROW = 4 * PAD;
-  __shared__ __attribute__((aligned(16))) float sq[DR_CH][ROW];
-  __shared__ __attribute__((aligned(16))) float sk[DR_CH][ROW];
-  __shared__ float sv[DR_CH][64];
-  __shared__ float sb[DR_CH], sg[DR_CH];
-  const int cols = blockDim.x >> 2;
-  const int cl = threadIdx.x >> 2, r = threadIdx.x & 3;
+  constexpr int PAD = RPT + 4;           // a part's rows in LDS, padded so that neighbouring parts lie in other banks
+  constexpr int ROW = R * PAD;
+  __shared__ __attribute__((aligned(16))) float sq[CH][ROW];
+  __shared__ __attribute__((aligned(16))) float sk[CH][ROW];
+  __shared__ float sv[CH][256 / R];
+  __shared__ float sb[CH], sg[CH];
+  const int cols = blockDim.x / R;
+  const int cl = threadIdx.x / R, r = threadIdx.x % R;
   const int j = blockIdx.x * cols + cl;
   const int h = blockIdx.y, seg = blockIdx.z;
   const int hk = h / (H / Hk);
@@ -149,50 +151,54 @@ __global__ __launch_bounds__(256) void delta_recurrence_kernel(
     const int i = r * RPT + ii;
     S[ii] = (st && active && i < dk) ? st[(size_t)i * dv + j] : 0.f;
   }
-  for (int c0 = 0; c0 < n; c0 += DR_CH) {
-    const int m = min(DR_CH, n - c0);
+  for (int c0 = 0; c0 < n; c0 += CH) {
+    const int m = min(CH, n - c0);
     __syncthreads();
-    for (int idx = threadIdx.x; idx < DR_CH * 4 * RPT; idx += blockDim.x) {
-      const int tt = idx / (4 * RPT), i = idx - tt * (4 * RPT);
+    for (int idx = threadIdx.x; idx < m * R * RPT; idx += blockDim.x) {
+      const int tt = idx / (R * RPT), i = idx - tt * (R * RPT);
       const int pos = (i / RPT) * PAD + (i % RPT);
-      const bool in = tt < m && i < dk;
+      const bool in = i < dk;
       const size_t src = ((size_t)(t0 + c0 + tt) * Hk + hk) * dk + i;
       sq[tt][pos] = in ? qn[src] : 0.f;
       sk[tt][pos] = in ? kn[src] : 0.f;
     }
-    for (int idx = threadIdx.x; idx < DR_CH * cols; idx += blockDim.x) {
+    for (int idx = threadIdx.x; idx < m * cols; idx += blockDim.x) {
       const int tt = idx / cols, c = idx - tt * cols;
       const int jj = blockIdx.x * cols + c;
-      sv[tt][c] = (tt < m && jj < dv) ? vc[((size_t)(t0 + c0 + tt) * H + h) * dv + jj] : 0.f;
+      sv[tt][c] = jj < dv ? vc[((size_t)(t0 + c0 + tt) * H + h) * dv + jj] : 0.f;
     }
-    if (threadIdx.x < DR_CH) {
+    if (threadIdx.x < m) {
       const int tt = threadIdx.x;
-      sb[tt] = tt < m ? beta[(size_t)(t0 + c0 + tt) * H + h] : 0.f;
-      sg[tt] = tt < m ? decay[(size_t)(t0 + c0 + tt) * H + h] : 1.f;
+      sb[tt] = beta[(size_t)(t0 + c0 + tt) * H + h];
+      sg[tt] = decay[(size_t)(t0 + c0 + tt) * H + h];
     }
     __syncthreads();
     for (int tt = 0; tt < m; ++tt) {
       const float g = sg[tt], b = sb[tt];
       const float* kr = &sk[tt][r * PAD];
       const float* qr = &sq[tt][r * PAD];
-      float kv = 0.f;
+      float kreg[RPT];
+      float kv[4] = {0.f, 0.f, 0.f, 0.f};          // four sums side by side: no chain of RPT dependent adds
 #pragma unroll
       for (int ii = 0; ii < RPT; ++ii) {
+        kreg[ii] = kr[ii];
         S[ii] *= g;
-        kv += S[ii] * kr[ii];
+        kv[ii & 3] += S[ii] * kreg[ii];
       }
-      kv += __shfl_xor(kv, 1, SA_WAVE);
-      kv += __shfl_xor(kv, 2, SA_WAVE);
-      const float u = b * (sv[tt][cl] - kv);
-      float oo = 0.f;
+      float kvs = (kv[0] + kv[1]) + (kv[2] + kv[3]);
+#pragma unroll
+      for (int off = 1; off < R; off <<= 1) kvs += __shfl_xor(kvs, off, SA_WAVE);
+      const float u = b * (sv[tt][cl] - kvs);
+      float oo[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ii = 0; ii < RPT; ++ii) {
-        S[ii] += kr[ii] * u;
-        oo += S[ii] * qr[ii];
+        S[ii] += kreg[ii] * u;
+        oo[ii & 3] += S[ii] * qr[ii];
       }
-      oo += __shfl_xor(oo, 1, SA_WAVE);
-      oo += __shfl_xor(oo, 2, SA_WAVE);
-      if (r == 0 && active) o[((size_t)(t0 + c0 + tt) * H + h) * dv + j] = oo;
+      float os = (oo[0] + oo[1]) + (oo[2] + oo[3]);
+#pragma unroll
+      for (int off = 1; off < R; off <<= 1) os += __shfl_xor(os, off, SA_WAVE);
+      if (r == 0 && active) o[((size_t)(t0 + c0 + tt) * H + h) * dv + j] = os;
     }
   }
   if (st && active) {
@@ -237,8 +243,8 @@ extern "C" long long sa_delta_rule_work_floats(int T, int H, int Hk, int dk, int
 extern "C" int sa_delta_rule(const void* z, int act_dtype, int zs, const float* conv_w, const float* ba,
                              const float* A_log, const float* dt_bias, const float* norm_w, float* state,
                              long long state_stride, const int* seg_of_token, const int* cu_q,
-                             const int* state_slots, float* work, void* y, float eps, int T, int B, int H, int Hk,
-                             int dk, int dv, int taps, hipStream_t stream) {
+                             const int* state_slots, float* work, void* y, float eps, int T, int B, int max_q_len,
+                             int H, int Hk, int dk, int dv, int taps, hipStream_t stream) {
   if (T <= 0 || B <= 0) return 0;
   if (H <= 0 || Hk <= 0 || H % Hk || dk <= 0 || dk > 256 || dv <= 0 || dv > 256 || taps < 1 || taps > DR_MAX_TAPS)
     return SA_ERR_ARG;
@@ -276,16 +282,30 @@ extern "C" int sa_delta_rule(const void* z, int act_dtype, int zs, const float* 
                          (size_t)state_stride, conv_off, cu_q, state_slots, C, taps);
     SA_LAUNCH_CHECK();
   }
-  {
+  if (max_q_len < 8) {
+    // single tokens (and portions of a few): 16 columns a wave
     const int waves = dv >= 64 ? 4 : (dv + 15) / 16;
     const int cols = 16 * waves;
     dim3 grid((dv + cols - 1) / cols, H, B), block(64 * waves);
 #define GO(RPT)                                                                                                 \
-  hipLaunchKernelGGL(delta_recurrence_kernel<RPT>, grid, block, 0, stream, qn, kn, vc, beta, decay, state,      \
-                     (size_t)state_stride, cu_q, state_slots, o, H, Hk, dk, dv)
+  hipLaunchKernelGGL((delta_recurrence_kernel<RPT, 4, 16>), grid, block, 0, stream, qn, kn, vc, beta, decay,    \
+                     state, (size_t)state_stride, cu_q, state_slots, o, H, Hk, dk, dv)
     if (dk <= 64) GO(16);
     else if (dk <= 128) GO(32);
     else GO(64);
+#undef GO
+    SA_LAUNCH_CHECK();
+  } else {
+    // prompt portions: 4 columns a wave, a step of the chain is a quarter as long
+    const int waves = dv >= 16 ? 4 : (dv + 3) / 4;
+    const int cols = 4 * waves;
+    dim3 grid((dv + cols - 1) / cols, H, B), block(64 * waves);
+#define GO(RPT)                                                                                                 \
+  hipLaunchKernelGGL((delta_recurrence_kernel<RPT, 16, 32>), grid, block, 0, stream, qn, kn, vc, beta, decay,   \
+                     state, (size_t)state_stride, cu_q, state_slots, o, H, Hk, dk, dv)
+    if (dk <= 64) GO(4);
+    else if (dk <= 128) GO(8);
+    else GO(16);
 #undef GO
     SA_LAUNCH_CHECK();
   }

@@ -12,7 +12,8 @@
 //   down      yk[perm[row], :] = Wd_e act[row, :]          (fp32)
 //   combine   y[t, :] = sum_k weights[t, k] yk[t top + k, :]  (+ sigmoid(sg[t]) * shared[t, :])
 //
-// Products: fp32 sums on the vector ALU over LDS tiles, storage types templated.
+// Products: bf16 on the matrix cores (moe_mfma_kernel); float32, and bf16 at sizes those do not take, as fp32
+// sums on the vector ALU over LDS tiles (storage types templated).
 #include "common.h"
 
 #define MOE_TM 32
@@ -65,7 +66,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
 // takes the next free row of its expert (the order inside an expert does not matter: a row's sums
 // do not depend on its place).
 // ---------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__ ids, int n, int E,
+__global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__ ids, int n, int E, int tile_rows,
                                                          int* __restrict__ offsets, int* __restrict__ cursor,
                                                          int* __restrict__ perm, int* __restrict__ tile_expert,
                                                          int* __restrict__ tile_row0, int* __restrict__ num_tiles) {
@@ -78,7 +79,7 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__
     for (int e = 0; e < E; ++e) {
       const int c = cursor[e];
       offsets[e] = run;
-      for (int r0 = 0; r0 < c; r0 += MOE_TM) {
+      for (int r0 = 0; r0 < c; r0 += tile_rows) {
         tile_expert[tiles] = e;
         tile_row0[tiles] = run + r0;
         ++tiles;
@@ -207,6 +208,132 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const TA* __restrict__ ac
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// The same two products on the matrix cores (bf16, K % 8 == 0): v_mfma_f32_16x16x32_bf16 computes the
+// transposed tile, operand "A" = 16 rows of the expert's matrix (lane l: row l % 16, k-slots 8 (l / 16) .. + 7),
+// operand "B" = 16 rows of activations, and lane l gets outputs n = 4 (l / 16) .. + 3 of activation row l % 16.
+// Weights and activations go from memory straight into registers, two steps of 32 along K ahead.
+//   KS == 1: tiles of up to 16 MT rows; the four waves of a workgroup own four groups of 16 weight rows
+//            and walk all of K (prompt portions: an expert's matrix is read once per 16 MT rows).
+//   KS == 4: tiles of up to 16 rows (MT 1); the four waves cut K between them and add through LDS in a
+//            fixed order (decode steps: few rows per expert, the chip is filled by cutting K and N).
+// GATE_UP: rows come from h by perm[row] / top, two matrices, act = silu(gate) * up in bf16.
+// else:    rows are act's own, one matrix, fp32 sums go to yk[perm[row]].
+// ---------------------------------------------------------------------------------------------
+typedef __bf16 moe_bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float moe_floatx4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int moe_u32x4_t __attribute__((ext_vector_type(4)));
+union MoeFrag {
+  moe_u32x4_t r;
+  moe_bf16x8_t v;
+};
+
+template <int MT, int KS, bool GATE_UP>
+__global__ __launch_bounds__(256) void moe_mfma_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W0,
+                                                       const bf16_t* __restrict__ W1, const int* __restrict__ offsets,
+                                                       const int* __restrict__ perm, const int* __restrict__ tile_expert,
+                                                       const int* __restrict__ tile_row0, const int* __restrict__ num_tiles,
+                                                       bf16_t* __restrict__ act, float* __restrict__ yk, int top, int N,
+                                                       int K) {
+  constexpr int RT = GATE_UP ? 2 : 1;
+  constexpr int KU = 2;
+  __shared__ float red[KS > 1 ? KS : 1][RT * MT * 4][64];
+  const int tile = blockIdx.x;
+  if (tile >= *num_tiles) return;
+  const int e = tile_expert[tile], row0 = tile_row0[tile];
+  const int rows = min(16 * MT, offsets[e + 1] - row0);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int g = lane >> 4, c = lane & 15;
+  const int n0 = (KS > 1 ? blockIdx.y : blockIdx.y * 4 + wave) * 16;
+  if (KS == 1 && n0 >= N) return;
+  const int nrow = min(n0 + c, N - 1);
+  const bf16_t* w0 = W0 + ((size_t)e * N + nrow) * K;
+  const bf16_t* w1 = GATE_UP ? W1 + ((size_t)e * N + nrow) * K : nullptr;
+  const bf16_t* arow[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int r = mt * 16 + c;
+    const int src = row0 + (r < rows ? r : 0);
+    arow[mt] = A + (size_t)(GATE_UP ? perm[src] / top : src) * K;
+  }
+  const int nchunks = (K + 31) >> 5;
+  const int per = (nchunks + KS - 1) / KS;
+  const int ch_begin = KS > 1 ? wave * per : 0;
+  const int ch_end = KS > 1 ? min(nchunks, ch_begin + per) : nchunks;
+  moe_floatx4_t acc[RT][MT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[rt][mt] = (moe_floatx4_t){0.f, 0.f, 0.f, 0.f};
+  const moe_u32x4_t zero = {0u, 0u, 0u, 0u};
+  for (int ch = ch_begin; ch < ch_end; ch += KU) {
+    MoeFrag wf[RT][KU], af[MT][KU];
+#pragma unroll
+    for (int u = 0; u < KU; ++u) {
+      const int k = min((ch + u) * 32 + g * 8, K - 8);
+      wf[0][u].r = *reinterpret_cast<const moe_u32x4_t*>(w0 + k);
+      if (GATE_UP) wf[RT - 1][u].r = *reinterpret_cast<const moe_u32x4_t*>(w1 + k);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) af[mt][u].r = *reinterpret_cast<const moe_u32x4_t*>(arow[mt] + k);
+    }
+    if (ch + KU > ch_end || (ch + KU) * 32 > K) {          // the last, partial round of the slice
+#pragma unroll
+      for (int u = 0; u < KU; ++u) {
+        const bool kin = (ch + u) < ch_end && (ch + u) * 32 + g * 8 < K;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) af[mt][u].r = kin ? af[mt][u].r : zero;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < KU; ++u)
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          acc[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[rt][u].v, af[mt][u].v, acc[rt][mt], 0, 0, 0);
+  }
+  if (KS > 1) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) red[wave][(rt * MT + mt) * 4 + r][lane] = acc[rt][mt][r];
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float sum = acc[rt][mt][r];
+          for (int w = 1; w < KS; ++w) sum += red[w][(rt * MT + mt) * 4 + r][lane];
+          acc[rt][mt][r] = sum;
+        }
+  }
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = mt * 16 + c;
+    if (m >= rows) continue;
+    const int n = n0 + 4 * g;
+    if (GATE_UP) {
+      bf16_t* dst = act + (size_t)(row0 + m) * N + n;
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (n + r < N) {
+          const float gv = acc[0][mt][r];
+          dst[r] = from_float<bf16_t>((gv / (1.f + expf(-gv))) * acc[RT - 1][mt][r]);
+        }
+    } else {
+      float* dst = yk + (size_t)perm[row0 + m] * N + n;
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (n + r < N) dst[r] = acc[0][mt][r];
+    }
+  }
+}
+
 // combine: grid (T).  shared: [parts, T, d] (TS), or null; sg: logits fp32, row stride ldz (null: no gate).
 template <typename TS>
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ yk, const float* __restrict__ wts,
@@ -228,7 +355,8 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
   }
 }
 
-extern "C" int sa_moe_max_tiles(int rows, int E) { return (rows + MOE_TM - 1) / MOE_TM + E; }
+// the most tiles a step can have, at the smallest tile (16 rows): what the scratch arrays are sized for
+extern "C" int sa_moe_max_tiles(int rows, int E) { return (rows + 15) / 16 + E; }
 
 extern "C" int sa_moe_route(const float* logits, int ldz, int* ids, float* wts, int T, int E, int top,
                             hipStream_t stream) {
@@ -241,6 +369,10 @@ extern "C" int sa_moe_route(const float* logits, int ldz, int* ids, float* wts, 
 }
 
 // ints: scratch of (E + 1) + E + n + 2 max_tiles + 1 int32 (offsets, cursor, perm, tile_expert, tile_row0, num_tiles)
+// with max_tiles = sa_moe_max_tiles(n, E).  bf16 with d and F multiples of 8 takes the matrix cores: up to
+// MOE_SMALL_ROWS rows (T top) in tiles of 16 with K cut over the waves, more in tiles of 64.
+#define MOE_SMALL_ROWS 1024
+
 extern "C" int sa_moe_experts(const void* h, int act_dtype, const int* ids, const void* Wg, const void* Wu,
                               const void* Wd, int* ints, void* act, float* yk, int T, int top, int E, int d, int F,
                               hipStream_t stream) {
@@ -254,10 +386,34 @@ extern "C" int sa_moe_experts(const void* h, int act_dtype, const int* ids, cons
   int* tile_expert = perm + n;
   int* tile_row0 = tile_expert + max_tiles;
   int* num_tiles = tile_row0 + max_tiles;
-  hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), 0, stream, ids, (int)n, E, offsets, cursor, perm,
+  const bool mfma = act_dtype == SA_BF16 && (d & 7) == 0 && (F & 7) == 0;
+  const bool small = n <= MOE_SMALL_ROWS;
+  const int tile_rows = mfma ? (small ? 16 : 64) : MOE_TM;
+  const int tiles = (int)((n + tile_rows - 1) / tile_rows) + E;
+  hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), 0, stream, ids, (int)n, E, tile_rows, offsets, cursor, perm,
                      tile_expert, tile_row0, num_tiles);
   SA_LAUNCH_CHECK();
-  dim3 g1(max_tiles, (F + MOE_TN - 1) / MOE_TN), g2(max_tiles, (d + MOE_TN - 1) / MOE_TN), block(256);
+  dim3 block(256);
+  if (mfma) {
+    const int per = small ? 16 : 64;          // weight rows a workgroup owns
+    dim3 g1(tiles, (F + per - 1) / per), g2(tiles, (d + per - 1) / per);
+    if (g1.y > 65535 || g2.y > 65535) return SA_ERR_ARG;
+#define GO(MT, KS)                                                                                                     \
+  do {                                                                                                                 \
+    hipLaunchKernelGGL((moe_mfma_kernel<MT, KS, true>), g1, block, 0, stream, (const bf16_t*)h, (const bf16_t*)Wg,     \
+                       (const bf16_t*)Wu, offsets, perm, tile_expert, tile_row0, num_tiles, (bf16_t*)act, nullptr,     \
+                       top, F, d);                                                                                     \
+    SA_LAUNCH_CHECK();                                                                                                 \
+    hipLaunchKernelGGL((moe_mfma_kernel<MT, KS, false>), g2, block, 0, stream, (const bf16_t*)act, (const bf16_t*)Wd,  \
+                       nullptr, offsets, perm, tile_expert, tile_row0, num_tiles, nullptr, yk, top, d, F);             \
+  } while (0)
+    if (small) GO(1, 4);
+    else GO(4, 1);
+#undef GO
+    SA_LAUNCH_CHECK();
+    return 0;
+  }
+  dim3 g1(tiles, (F + MOE_TN - 1) / MOE_TN), g2(tiles, (d + MOE_TN - 1) / MOE_TN);
   if (g1.y > 65535 || g2.y > 65535) return SA_ERR_ARG;
   if (act_dtype == SA_F32) {
     hipLaunchKernelGGL(moe_gate_up_kernel<float>, g1, block, 0, stream, (const float*)h, (const float*)Wg,

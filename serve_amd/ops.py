@@ -462,7 +462,8 @@ def delta_rule(z: torch.Tensor, conv_w: torch.Tensor, ba: torch.Tensor, A_log: t
     _ret(lib.sa_delta_rule(_ptr(z), c_int(_code(z)), c_int(z.shape[1]), _ptr(conv_w), _ptr(ba), _ptr(A_log),
                            _ptr(dt_bias), _ptr(norm_w), _ptr(state), ctypes.c_longlong(state.shape[1]),
                            _ptr(ctx.seg_of_token), _ptr(ctx.cu_q), _ptr(ctx.state_slots), _ptr(work), _ptr(y),
-                           c_float(eps), c_int(T), c_int(B), c_int(H), c_int(Hk), c_int(dk), c_int(dv), c_int(taps),
+                           c_float(eps), c_int(T), c_int(B), c_int(int(getattr(ctx, "max_q_len", T) or T)), c_int(H), c_int(Hk), c_int(dk),
+                           c_int(dv), c_int(taps),
                            _stream()), "delta_rule")
     return y
 

@@ -264,20 +264,21 @@ def test_route_picks_the_largest_and_weights_them_among_themselves(experts, top)
     assert torch.allclose(w.double(), torch.softmax(vals, -1), atol=1e-6)
 
 
+@pytest.mark.parametrize("T,d,F", [(45, 72, 40), (45, 75, 42), (400, 64, 48)])   # few rows; sizes the matrix cores do not take; many rows
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_experts_against_one_by_one(dtype):
+def test_experts_against_one_by_one(dtype, T, d, F):
     from serve_amd import ops
     torch.manual_seed(3)
-    T, d, F, E, top = 45, 72, 40, 7, 3
+    E, top = 7, 3
     h = torch.randn(T, d, device="cuda").to(dtype)
     wg, wu = (torch.randn(E, F, d, device="cuda") * 0.2).to(dtype), (torch.randn(E, F, d, device="cuda") * 0.2).to(dtype)
     wd = (torch.randn(E, d, F, device="cuda") * 0.2).to(dtype)
     ids = torch.stack([torch.randperm(E, device="cuda")[:top] for _ in range(T)]).int().contiguous()
-    ids[5:40] = ids[4]                                   # many rows for few experts: more than one tile of rows
+    ids[5: T - 5] = ids[4]                               # many rows for few experts: more than one tile of rows
     yk = torch.empty(T * top, d, dtype=torch.float32, device="cuda")
     ops.moe_experts(h, ids, wg, wu, wd, yk)
     hd = h.double()
-    for t in range(T):
+    for t in list(range(0, T, 7)) + [4, 5, T - 6, T - 5, T - 1]:
         for k in range(top):
             e = int(ids[t, k])
             a = torch.nn.functional.silu(hd[t] @ wg[e].double().t()) * (hd[t] @ wu[e].double().t())
@@ -287,8 +288,9 @@ def test_experts_against_one_by_one(dtype):
             assert torch.allclose(yk[t * top + k].double(), want, atol=2e-4 if dtype == torch.float32 else 2e-2, rtol=1e-3)
 
 
+@pytest.mark.parametrize("longest", [1, 64])      # which shape of the recurrence kernel runs: single tokens, prompt portions
 @pytest.mark.parametrize("dk,dv,heads,kv_heads,taps", [(16, 24, 4, 2, 3), (72, 80, 2, 1, 4), (200, 8, 1, 1, 1), (33, 130, 3, 3, 2)])
-def test_delta_rule_kernels_in_two_steps(dk, dv, heads, kv_heads, taps):
+def test_delta_rule_kernels_in_two_steps(dk, dv, heads, kv_heads, taps, longest):
     """The kernels over two steps of two segments (one of them a single token) against the plain
     recurrence over the whole sequences: the state and the convolution's last inputs carry over."""
     from types import SimpleNamespace
@@ -325,7 +327,7 @@ def test_delta_rule_kernels_in_two_steps(dk, dv, heads, kv_heads, taps):
         zs = torch.cat([z[r][at[r]: at[r] + n[r]] for r in range(2)])
         bs = torch.cat([ba[r][at[r]: at[r] + n[r]] for r in range(2)])
         T = zs.shape[0]
-        ctx = SimpleNamespace(num_tokens=T, num_segments=2,
+        ctx = SimpleNamespace(num_tokens=T, num_segments=2, max_q_len=longest,
                               seg_of_token=torch.tensor([0] * n[0] + [1] * n[1], dtype=torch.int32, device="cuda"),
                               cu_q=torch.tensor([0, n[0], T], dtype=torch.int32, device="cuda"),
                               state_slots=torch.tensor([2, 0], dtype=torch.int32, device="cuda"))

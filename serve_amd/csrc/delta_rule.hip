@@ -124,6 +124,25 @@ __global__ __launch_bounds__(256) void delta_conv_state_kernel(
 // a step is what counts.  The tokens of a segment come through LDS in chunks of CH; a segment's state is
 // read once and written once.
 // ---------------------------------------------------------------------------------------------
+// The sum of v over groups of R neighbouring lanes (R = 4 or 16), in every lane of the group, by data-parallel
+// moves inside a row of 16 lanes: neighbours, pairs of neighbours, then the mirrored half and the mirrored row
+// (every lane of a group of four, then of eight, already holds its group's sum, so mirrors serve as well as swaps).
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+template <int R>
+__device__ __forceinline__ float lanes_sum(float v) {
+  static_assert(R == 4 || R == 16, "groups of 4 or 16 lanes");
+  v += dpp_move<0xB1>(v);          // quad_perm [1, 0, 3, 2]
+  v += dpp_move<0x4E>(v);          // quad_perm [2, 3, 0, 1]
+  if (R == 16) {
+    v += dpp_move<0x141>(v);       // row_half_mirror
+    v += dpp_move<0x140>(v);       // row_mirror
+  }
+  return v;
+}
+
 template <int RPT, int R, int CH>
 __global__ __launch_bounds__(256) void delta_recurrence_kernel(
     const float* __restrict__ qn, const float* __restrict__ kn, const float* __restrict__ vc,
@@ -173,32 +192,41 @@ __global__ __launch_bounds__(256) void delta_recurrence_kernel(
       sg[tt] = decay[(size_t)(t0 + c0 + tt) * H + h];
     }
     __syncthreads();
+    // One pass over the thread's rows a token: with Sd = g S, a = Sd^T k and c = Sd^T q are summed side by
+    // side (and k.q with them), u = beta (v - a), the read-out of the updated state is c + u (k.q), and
+    // S = Sd + k u.  The three sums cross the R lanes together; the next token's k and q are fetched from
+    // LDS before this token's sums are awaited.
+    float kreg[RPT], qreg[RPT];
+#pragma unroll
+    for (int ii = 0; ii < RPT; ++ii) {
+      kreg[ii] = sk[0][r * PAD + ii];
+      qreg[ii] = sq[0][r * PAD + ii];
+    }
     for (int tt = 0; tt < m; ++tt) {
-      const float g = sg[tt], b = sb[tt];
-      const float* kr = &sk[tt][r * PAD];
-      const float* qr = &sq[tt][r * PAD];
-      float kreg[RPT];
-      float kv[4] = {0.f, 0.f, 0.f, 0.f};          // four sums side by side: no chain of RPT dependent adds
+      const float g = sg[tt], b = sb[tt], vj = sv[tt][cl];
+      float a4[4] = {0.f, 0.f, 0.f, 0.f}, c4[4] = {0.f, 0.f, 0.f, 0.f}, p4[4] = {0.f, 0.f, 0.f, 0.f};
+      float kcur[RPT];
 #pragma unroll
       for (int ii = 0; ii < RPT; ++ii) {
-        kreg[ii] = kr[ii];
+        kcur[ii] = kreg[ii];
         S[ii] *= g;
-        kv[ii & 3] += S[ii] * kreg[ii];
+        a4[ii & 3] += S[ii] * kreg[ii];
+        c4[ii & 3] += S[ii] * qreg[ii];
+        p4[ii & 3] += kreg[ii] * qreg[ii];
       }
-      float kvs = (kv[0] + kv[1]) + (kv[2] + kv[3]);
-#pragma unroll
-      for (int off = 1; off < R; off <<= 1) kvs += __shfl_xor(kvs, off, SA_WAVE);
-      const float u = b * (sv[tt][cl] - kvs);
-      float oo[4] = {0.f, 0.f, 0.f, 0.f};
+      const int nx = min(tt + 1, m - 1);
 #pragma unroll
       for (int ii = 0; ii < RPT; ++ii) {
-        S[ii] += kreg[ii] * u;
-        oo[ii & 3] += S[ii] * qr[ii];
+        kreg[ii] = sk[nx][r * PAD + ii];
+        qreg[ii] = sq[nx][r * PAD + ii];
       }
-      float os = (oo[0] + oo[1]) + (oo[2] + oo[3]);
+      const float a = lanes_sum<R>((a4[0] + a4[1]) + (a4[2] + a4[3]));
+      const float c = lanes_sum<R>((c4[0] + c4[1]) + (c4[2] + c4[3]));
+      const float kq = lanes_sum<R>((p4[0] + p4[1]) + (p4[2] + p4[3]));
+      const float u = b * (vj - a);
 #pragma unroll
-      for (int off = 1; off < R; off <<= 1) os += __shfl_xor(os, off, SA_WAVE);
-      if (r == 0 && active) o[((size_t)(t0 + c0 + tt) * H + h) * dv + j] = os;
+      for (int ii = 0; ii < RPT; ++ii) S[ii] += kcur[ii] * u;
+      if (r == 0 && active) o[((size_t)(t0 + c0 + tt) * H + h) * dv + j] = c + u * kq;
     }
   }
   if (st && active) {

@@ -110,10 +110,17 @@ __global__ __launch_bounds__(256) void head_linear_kernel(const TA* __restrict__
     }
     __syncthreads();
     if (n < N) {
-      for (int k = 0; k < kc; ++k) {
-        const float wv = to_float(Wh[(size_t)(k0 + k) * N + n]);
+      // eight rows of W at a time, their loads issued together (a row beyond the chunk: clamped and dropped)
+      for (int k = 0; k < kc; k += 8) {
+        float wv[8];
 #pragma unroll
-        for (int tt = 0; tt < HL_TT; ++tt) acc[tt] += sin_[tt][k] * wv;
+        for (int u = 0; u < 8; ++u) wv[u] = to_float(Wh[(size_t)(k0 + min(k + u, kc - 1)) * N + n]);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const float wu = k + u < kc ? wv[u] : 0.f;
+#pragma unroll
+          for (int tt = 0; tt < HL_TT; ++tt) acc[tt] += sin_[tt][min(k + u, HL_KC - 1)] * wu;
+        }
       }
     }
   }

@@ -335,7 +335,9 @@ __global__ __launch_bounds__(256) void moe_mfma_kernel(const bf16_t* __restrict_
 }
 
 // combine: grid (T).  shared: [parts, T, d] (TS), or null; sg: logits fp32, row stride ldz (null: no gate).
-template <typename TS>
+// TOPMAX / PMAX: upper bounds of `top` / `parts` (0: any number, in a loop): with bounds, all loads of an output
+// are issued before anything is added (rows beyond the bounds are read from a clamped place and dropped).
+template <typename TS, int TOPMAX, int PMAX>
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ yk, const float* __restrict__ wts,
                                                           const TS* __restrict__ shared, int parts, size_t part_stride,
                                                           const float* __restrict__ sg, int ldz, float* __restrict__ y,
@@ -343,13 +345,33 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
   const int t = blockIdx.x;
   float gate = 1.f;
   if (shared && sg) gate = 1.f / (1.f + expf(-sg[(size_t)t * ldz]));
+  if (TOPMAX > 0) {
+    float wk[TOPMAX > 0 ? TOPMAX : 1];
+#pragma unroll
+    for (int k = 0; k < TOPMAX; ++k) wk[k] = k < top ? wts[(size_t)t * top + k] : 0.f;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+      float a[TOPMAX > 0 ? TOPMAX : 1], sp[PMAX];
+#pragma unroll
+      for (int k = 0; k < TOPMAX; ++k) a[k] = yk[((size_t)t * top + min(k, top - 1)) * d + i];
+#pragma unroll
+      for (int p = 0; p < PMAX; ++p) sp[p] = shared ? to_float(shared[min(p, parts - 1) * part_stride + (size_t)t * d + i]) : 0.f;
+      float v = 0.f;
+#pragma unroll
+      for (int k = 0; k < TOPMAX; ++k) v += wk[k] * a[k];
+      float sh = 0.f;
+#pragma unroll
+      for (int p = 0; p < PMAX; ++p) sh += p < parts ? sp[p] : 0.f;
+      y[(size_t)t * d + i] = shared ? v + gate * sh : v;
+    }
+    return;
+  }
   for (int i = threadIdx.x; i < d; i += blockDim.x) {
     float v = 0.f;
     for (int k = 0; k < top; ++k) v += wts[(size_t)t * top + k] * yk[((size_t)t * top + k) * d + i];
     if (shared) {
-      float s = 0.f;
-      for (int p = 0; p < parts; ++p) s += to_float(shared[p * part_stride + (size_t)t * d + i]);
-      v += gate * s;
+      float sh = 0.f;
+      for (int p = 0; p < parts; ++p) sh += to_float(shared[p * part_stride + (size_t)t * d + i]);
+      v += gate * sh;
     }
     y[(size_t)t * d + i] = v;
   }
@@ -440,12 +462,18 @@ extern "C" int sa_moe_combine(const float* yk, const float* wts, const void* sha
   if (top <= 0 || d <= 0 || parts < 1) return SA_ERR_ARG;
   const size_t part_stride = (size_t)T * d;
   dim3 grid(T), block(d >= 256 ? 256 : 64);
-  if (!shared || shared_dtype == SA_F32)
-    hipLaunchKernelGGL(moe_combine_kernel<float>, grid, block, 0, stream, yk, wts, (const float*)shared, parts,
-                       part_stride, sg, ldz, y, top, d);
-  else if (shared_dtype == SA_BF16 && parts == 1)
-    hipLaunchKernelGGL(moe_combine_kernel<bf16_t>, grid, block, 0, stream, yk, wts, (const bf16_t*)shared, parts,
-                       part_stride, sg, ldz, y, top, d);
+#define GO(TS, TOPMAX, PMAX)                                                                                       \
+  hipLaunchKernelGGL((moe_combine_kernel<TS, TOPMAX, PMAX>), grid, block, 0, stream, yk, wts, (const TS*)shared,     \
+                     parts, part_stride, sg, ldz, y, top, d)
+  const bool bounded = top <= 8 && parts <= 8;
+  if (!shared || shared_dtype == SA_F32) {
+    if (bounded) GO(float, 8, 8);
+    else GO(float, 0, 1);
+  } else if (shared_dtype == SA_BF16 && parts == 1) {
+    if (bounded) GO(bf16_t, 8, 1);
+    else GO(bf16_t, 0, 1);
+  }
+#undef GO
   else return SA_ERR_UNSUPPORTED;
   SA_LAUNCH_CHECK();
   return 0;

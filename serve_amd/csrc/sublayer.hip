@@ -66,6 +66,74 @@ __global__ __launch_bounds__(256) void output_norm_add_kernel(float* __restrict_
   }
 }
 
+// The same for d % 4 == 0 and d <= 8192: 16-byte vectors, and every load of a row (the parts of y, x, w, s) is
+// issued before anything is added, so that a row costs one trip to memory.  PMAX: upper bound of `parts`; a part
+// beyond `parts` is read from a clamped address and dropped.
+__device__ __forceinline__ float4 ld4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 ld4(const bf16_t* p) {
+  const uint2 u = *reinterpret_cast<const uint2*>(p);
+  return make_float4(bf16_bits_to_float(u.x & 0xffffu), bf16_bits_to_float(u.x >> 16),
+                     bf16_bits_to_float(u.y & 0xffffu), bf16_bits_to_float(u.y >> 16));
+}
+__device__ __forceinline__ void st4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void st4(bf16_t* p, float4 v) {
+  uint2 u;
+  u.x = (uint32_t)float_to_bf16_bits(v.x) | ((uint32_t)float_to_bf16_bits(v.y) << 16);
+  u.y = (uint32_t)float_to_bf16_bits(v.z) | ((uint32_t)float_to_bf16_bits(v.w) << 16);
+  *reinterpret_cast<uint2*>(p) = u;
+}
+
+template <typename TA, typename TD, int PMAX, int NG>
+__global__ __launch_bounds__(256) void output_norm_add_vec_kernel(float* __restrict__ x, const TD* __restrict__ y,
+                                                                  int parts, size_t part_stride,
+                                                                  const float* __restrict__ w,
+                                                                  const float* __restrict__ s, TA* __restrict__ h,
+                                                                  float eps, int d) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x;
+  float* xr = x + (size_t)t * d;
+  const TD* yr = y + (size_t)t * d;
+  const int groups = d >> 2;
+  float4 v[NG], xv[NG], wv[NG], sv[NG];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < NG; ++k) {
+    const int gi = threadIdx.x + k * 256;
+    const int i = min(gi, groups - 1) * 4;
+    float4 a[PMAX];
+#pragma unroll
+    for (int p = 0; p < PMAX; ++p) a[p] = ld4(yr + (size_t)min(p, parts - 1) * part_stride + i);
+    xv[k] = ld4(xr + i);
+    wv[k] = ld4(w + i);
+    sv[k] = ld4(s + i);
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int p = 0; p < PMAX; ++p) {
+      const float on = p < parts ? 1.f : 0.f;
+      acc.x += on * a[p].x; acc.y += on * a[p].y; acc.z += on * a[p].z; acc.w += on * a[p].w;
+    }
+    v[k] = acc;
+    const float in = gi < groups ? 1.f : 0.f;
+    ss += in * (acc.x * acc.x + acc.y * acc.y + acc.z * acc.z + acc.w * acc.w);
+  }
+  ss = block_sum(ss, scratch);
+  const float rs = 1.0f / sqrtf(ss / (float)d + eps);
+#pragma unroll
+  for (int k = 0; k < NG; ++k) {
+    const int gi = threadIdx.x + k * 256;
+    if (gi < groups) {
+      const int i = gi * 4;
+      float4 nx;
+      nx.x = xv[k].x + ((v[k].x * rs) * wv[k].x) * sv[k].x;
+      nx.y = xv[k].y + ((v[k].y * rs) * wv[k].y) * sv[k].y;
+      nx.z = xv[k].z + ((v[k].z * rs) * wv[k].z) * sv[k].z;
+      nx.w = xv[k].w + ((v[k].w * rs) * wv[k].w) * sv[k].w;
+      st4(xr + i, nx);
+      if (h) st4(h + (size_t)t * d + i, nx);
+    }
+  }
+}
+
 extern "C" int sa_output_norm_add(float* x, const void* y, int y_dtype, int parts, const float* w, const float* s,
                                   void* h, int act_dtype, float eps, int T, int d, hipStream_t stream) {
   if (T <= 0) return 0;
@@ -75,6 +143,33 @@ extern "C" int sa_output_norm_add(float* x, const void* y, int y_dtype, int part
   if (y && parts > 1 && y_dtype != SA_F32) return SA_ERR_UNSUPPORTED;
   const size_t part_stride = (size_t)T * d;
   dim3 grid(T), block(d >= 1024 ? 256 : (d >= 256 ? 128 : 64));
+  if (y && (d & 3) == 0 && d >= 256 && d <= 8192 && parts <= 8) {
+    const int ng = (d / 4 + 255) / 256;          // groups of four a thread, 1 .. 8
+#define GOV(TA, TD, PMAX, NG)                                                                                   \
+  hipLaunchKernelGGL((output_norm_add_vec_kernel<TA, TD, PMAX, NG>), grid, dim3(256), 0, stream, x,             \
+                     (const TD*)y, parts, part_stride, w, s, (TA*)h, eps, d)
+#define GON(TA, TD, PMAX)                                                                                       \
+  do {                                                                                                          \
+    if (ng <= 1) GOV(TA, TD, PMAX, 1);                                                                          \
+    else if (ng <= 2) GOV(TA, TD, PMAX, 2);                                                                     \
+    else if (ng <= 4) GOV(TA, TD, PMAX, 4);                                                                     \
+    else GOV(TA, TD, PMAX, 8);                                                                                  \
+  } while (0)
+#define GOP(TA, TD)                                                                                             \
+  do {                                                                                                          \
+    if (parts == 1) GON(TA, TD, 1);                                                                             \
+    else if (parts <= 4) GON(TA, TD, 4);                                                                        \
+    else GON(TA, TD, 8);                                                                                        \
+  } while (0)
+    if (act_dtype == SA_F32) GOP(float, float);
+    else if (act_dtype == SA_BF16) { if (y_dtype == SA_F32) GOP(bf16_t, float); else GON(bf16_t, bf16_t, 1); }
+    else return SA_ERR_UNSUPPORTED;
+#undef GOP
+#undef GON
+#undef GOV
+    SA_LAUNCH_CHECK();
+    return 0;
+  }
 #define GO(TA, TD)                                                                                          \
   hipLaunchKernelGGL((output_norm_add_kernel<TA, TD>), grid, block, 0, stream, x, (const TD*)y, parts,      \
                      part_stride, w, s, (TA*)h, eps, d)

@@ -239,6 +239,143 @@ __global__ __launch_bounds__(256) void delta_recurrence_kernel(
 }
 
 // ---------------------------------------------------------------------------------------------
+// (3b) the recurrence for prompt portions, four tokens a pass.  With S0 the state before tokens 0..3 of a
+// block, G_i = g_0 .. g_i and r_li = g_(l+1) .. g_i:
+//     a_i = G_i S0^T k_i + sum_(l<i)  r_li u_l (k_l . k_i)          u_i = beta_i (v_i - a_i)
+//     o_i = G_i S0^T q_i + sum_(l<=i) r_li u_l (k_l . q_i)          S  = G_3 S0 + sum_l r_l3 k_l u_l^T
+// so one pass over the thread's rows gives the eight sums S0^T k_i, S0^T q_i, one exchange between the lanes
+// carries all eight, the four u_i follow from scalars alone, and a second pass writes the new state: the
+// chain of dependent steps is a quarter as long as token by token.  The products k_l . k_i and k_l . q_i do
+// not depend on the state: they are taken once per chunk, from LDS, for all columns.  A block that the
+// segment's end cuts short is filled with tokens that change nothing (k = q = 0, beta = 0, g = 1).
+// ---------------------------------------------------------------------------------------------
+template <int RPT, int CH>
+__global__ __launch_bounds__(256) void delta_recurrence_block_kernel(
+    const float* __restrict__ qn, const float* __restrict__ kn, const float* __restrict__ vc,
+    const float* __restrict__ beta, const float* __restrict__ decay, float* __restrict__ state,
+    size_t state_stride, const int* __restrict__ cu_q, const int* __restrict__ state_slots,
+    float* __restrict__ o, int H, int Hk, int dk, int dv) {
+  constexpr int R = 16;
+  constexpr int PAD = RPT + 4;
+  constexpr int ROW = R * PAD;
+  constexpr int NB = CH / 4;
+  static_assert(CH % 4 == 0, "chunks are whole blocks of four");
+  __shared__ __attribute__((aligned(16))) float sq[CH][ROW];
+  __shared__ __attribute__((aligned(16))) float sk[CH][ROW];
+  __shared__ float sv[CH][16];
+  __shared__ float sb[CH], sg[CH];
+  __shared__ float skk[NB][6];           // k_l . k_i, l < i:  (0,1) (0,2) (0,3) (1,2) (1,3) (2,3)
+  __shared__ float skq[NB][10];          // k_l . q_i, l <= i: (0,0) (0,1) (0,2) (0,3) (1,1) (1,2) (1,3) (2,2) (2,3) (3,3)
+  const int cols = blockDim.x / R;
+  const int cl = threadIdx.x / R, r = threadIdx.x % R;
+  const int j = blockIdx.x * cols + cl;
+  const int h = blockIdx.y, seg = blockIdx.z;
+  const int hk = h / (H / Hk);
+  const bool active = j < dv;
+  const int slot = state_slots[seg];
+  const int t0 = cu_q[seg], n = cu_q[seg + 1] - t0;
+  float* st = slot >= 0 ? state + (size_t)slot * state_stride + (size_t)h * dk * dv : nullptr;
+  float S[RPT];
+#pragma unroll
+  for (int ii = 0; ii < RPT; ++ii) {
+    const int i = r * RPT + ii;
+    S[ii] = (st && active && i < dk) ? st[(size_t)i * dv + j] : 0.f;
+  }
+  for (int c0 = 0; c0 < n; c0 += CH) {
+    const int m = min(CH, n - c0);
+    const int mpad = (m + 3) & ~3;
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < mpad * R * RPT; idx += blockDim.x) {
+      const int tt = idx / (R * RPT), i = idx - tt * (R * RPT);
+      const int pos = (i / RPT) * PAD + (i % RPT);
+      const bool in = tt < m && i < dk;
+      const size_t src = ((size_t)(t0 + c0 + min(tt, m - 1)) * Hk + hk) * dk + min(i, dk - 1);
+      const float qv = qn[src], kv = kn[src];
+      sq[tt][pos] = in ? qv : 0.f;
+      sk[tt][pos] = in ? kv : 0.f;
+    }
+    for (int idx = threadIdx.x; idx < mpad * cols; idx += blockDim.x) {
+      const int tt = idx / cols, c = idx - tt * cols;
+      const int jj = blockIdx.x * cols + c;
+      sv[tt][c] = (tt < m && jj < dv) ? vc[((size_t)(t0 + c0 + tt) * H + h) * dv + jj] : 0.f;
+    }
+    if (threadIdx.x < mpad) {
+      const int tt = threadIdx.x;
+      sb[tt] = tt < m ? beta[(size_t)(t0 + c0 + tt) * H + h] : 0.f;
+      sg[tt] = tt < m ? decay[(size_t)(t0 + c0 + tt) * H + h] : 1.f;
+    }
+    __syncthreads();
+    // the state-free products of every block of the chunk: sixteen a block, one per group of R lanes and pass
+    // (a lane sums its part of the rows, the group adds up)
+    for (int id = cl; id < (mpad / 4) * 16; id += cols) {
+      const int blk = id >> 4, which = id & 15;
+      const int l = (int)((0xe9500940ull >> (2 * which)) & 3), i = (int)((0xfb9e4fb9ull >> (2 * which)) & 3);
+      const float* kl = &sk[blk * 4 + l][r * PAD];
+      const float* xi = which >= 6 ? &sq[blk * 4 + i][r * PAD] : &sk[blk * 4 + i][r * PAD];
+      float dsum = 0.f;
+#pragma unroll
+      for (int ii = 0; ii < RPT; ++ii) dsum += kl[ii] * xi[ii];
+      dsum = lanes_sum<R>(dsum);
+      if (r == 0) {
+        if (which >= 6) skq[blk][which - 6] = dsum;
+        else skk[blk][which] = dsum;
+      }
+    }
+    __syncthreads();
+    for (int bb = 0; bb < mpad / 4; ++bb) {
+      const int tb = bb * 4;
+      float A[4] = {0.f, 0.f, 0.f, 0.f}, C[4] = {0.f, 0.f, 0.f, 0.f};
+      float kr[4][RPT];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int ii = 0; ii < RPT; ++ii) {
+          kr[i][ii] = sk[tb + i][r * PAD + ii];
+          A[i] += S[ii] * kr[i][ii];
+          C[i] += S[ii] * sq[tb + i][r * PAD + ii];
+        }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        A[i] = lanes_sum<R>(A[i]);
+        C[i] = lanes_sum<R>(C[i]);
+      }
+      const float g0 = sg[tb], g1 = sg[tb + 1], g2 = sg[tb + 2], g3 = sg[tb + 3];
+      const float G0 = g0, G1 = g0 * g1, G2 = G1 * g2, G3 = G2 * g3;
+      const float r01 = g1, r02 = g1 * g2, r03 = r02 * g3, r12 = g2, r13 = g2 * g3, r23 = g3;
+      const float* kk = skk[bb];
+      const float* kq = skq[bb];
+      const float u0 = sb[tb] * (sv[tb][cl] - G0 * A[0]);
+      const float u1 = sb[tb + 1] * (sv[tb + 1][cl] - (G1 * A[1] + r01 * u0 * kk[0]));
+      const float u2 = sb[tb + 2] * (sv[tb + 2][cl] - (G2 * A[2] + r02 * u0 * kk[1] + r12 * u1 * kk[3]));
+      const float u3 = sb[tb + 3] * (sv[tb + 3][cl] - (G3 * A[3] + r03 * u0 * kk[2] + r13 * u1 * kk[4] + r23 * u2 * kk[5]));
+      const float o0 = G0 * C[0] + u0 * kq[0];
+      const float o1 = G1 * C[1] + r01 * u0 * kq[1] + u1 * kq[4];
+      const float o2 = G2 * C[2] + r02 * u0 * kq[2] + r12 * u1 * kq[5] + u2 * kq[7];
+      const float o3 = G3 * C[3] + r03 * u0 * kq[3] + r13 * u1 * kq[6] + r23 * u2 * kq[8] + u3 * kq[9];
+      const float w0 = r03 * u0, w1 = r13 * u1, w2 = r23 * u2;
+#pragma unroll
+      for (int ii = 0; ii < RPT; ++ii)
+        S[ii] = G3 * S[ii] + ((w0 * kr[0][ii] + w1 * kr[1][ii]) + (w2 * kr[2][ii] + u3 * kr[3][ii]));
+      if (r == 0 && active) {
+        float* op = o + ((size_t)(t0 + c0 + tb) * H + h) * dv + j;
+        const size_t os = (size_t)H * dv;
+        if (tb < m) op[0] = o0;
+        if (tb + 1 < m) op[os] = o1;
+        if (tb + 2 < m) op[2 * os] = o2;
+        if (tb + 3 < m) op[3 * os] = o3;
+      }
+    }
+  }
+  if (st && active) {
+#pragma unroll
+    for (int ii = 0; ii < RPT; ++ii) {
+      const int i = r * RPT + ii;
+      if (i < dk) st[(size_t)i * dv + j] = S[ii];
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
 // (4) y[t, h, :] = o[t, h, :] / sqrt(mean(o^2) + eps) * w * silu(gate[t, h, :]); gate is a block of
 // columns of z.  A wave per (token, head).
 // ---------------------------------------------------------------------------------------------
@@ -324,12 +461,12 @@ extern "C" int sa_delta_rule(const void* z, int act_dtype, int zs, const float* 
 #undef GO
     SA_LAUNCH_CHECK();
   } else {
-    // prompt portions: 4 columns a wave, a step of the chain is a quarter as long
+    // prompt portions: 4 columns a wave, four tokens a pass over the state
     const int waves = dv >= 16 ? 4 : (dv + 3) / 4;
     const int cols = 4 * waves;
     dim3 grid((dv + cols - 1) / cols, H, B), block(64 * waves);
 #define GO(RPT)                                                                                                 \
-  hipLaunchKernelGGL((delta_recurrence_kernel<RPT, 16, 32>), grid, block, 0, stream, qn, kn, vc, beta, decay,   \
+  hipLaunchKernelGGL((delta_recurrence_block_kernel<RPT, 32>), grid, block, 0, stream, qn, kn, vc, beta, decay, \
                      state, (size_t)state_stride, cu_q, state_slots, o, H, Hk, dk, dv)
     if (dk <= 64) GO(4);
     else if (dk <= 128) GO(8);

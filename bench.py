@@ -251,9 +251,14 @@ def designs(args) -> int:
             steps = args.steps
             prompt_len = context - steps - 8 - 3 - head_start(engine, b, context)
             dt, mean_ctx = decode_run(engine, b, prompt_len, 8, steps, seed=10 + b)
-            nbytes = weight_bytes(engine.model, item) + b * kv_bytes(engine.model, mean_ctx, item)
+            # the weights a step of b tokens reads (with experts: as many as b tokens can choose), the cache, and
+            # the recurrent state of every request, read and written
+            elements, _ = engine.model.step_cost(b, logit_rows=b)
+            state = sum(4 * 2 * b * int(__import__("math").prod(sr.shape)) for sr in engine.model.state_requests() if sr)
+            nbytes = item * elements + b * kv_bytes(engine.model, mean_ctx, item) + state
             out[f"decode_b{b}"] = {"ms_per_step": round(dt / steps * 1e3, 4), "tokens_per_s": round(b * steps / dt, 1),
-                                   "context": int(mean_ctx), "TB_per_s": round(nbytes / (dt / steps) / 1e12, 3)}
+                                   "context": int(mean_ctx), "GB_per_step": round(nbytes / 1e9, 3),
+                                   "TB_per_s": round(nbytes / (dt / steps) / 1e12, 3)}
         print(json.dumps(out), flush=True)
         del engine
         torch.cuda.empty_cache()

@@ -110,17 +110,10 @@ __global__ __launch_bounds__(256) void head_linear_kernel(const TA* __restrict__
     }
     __syncthreads();
     if (n < N) {
-      // eight rows of W at a time, their loads issued together (a row beyond the chunk: clamped and dropped)
-      for (int k = 0; k < kc; k += 8) {
-        float wv[8];
+      for (int k = 0; k < kc; ++k) {
+        const float wv = to_float(Wh[(size_t)(k0 + k) * N + n]);
 #pragma unroll
-        for (int u = 0; u < 8; ++u) wv[u] = to_float(Wh[(size_t)(k0 + min(k + u, kc - 1)) * N + n]);
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const float wu = k + u < kc ? wv[u] : 0.f;
-#pragma unroll
-          for (int tt = 0; tt < HL_TT; ++tt) acc[tt] += sin_[tt][min(k + u, HL_KC - 1)] * wu;
-        }
+        for (int tt = 0; tt < HL_TT; ++tt) acc[tt] += sin_[tt][k] * wv;
       }
     }
   }
@@ -131,10 +124,60 @@ __global__ __launch_bounds__(256) void head_linear_kernel(const TA* __restrict__
   }
 }
 
+// The same for few tokens (single decoded tokens): a workgroup per (token, head), the four waves cut K between
+// them and add through LDS in a fixed order, a lane owns an output column and fetches sixteen rows of W at a time,
+// so that the whole product is a few trips to memory.  K <= HL_SMALL_K.
+#define HL_SMALL_K 1024
+
+template <typename TA>
+__global__ __launch_bounds__(256) void head_linear_small_kernel(const TA* __restrict__ in, int is, int ihs,
+                                                                const TA* __restrict__ W, TA* __restrict__ out, int os,
+                                                                int ohs, int K, int N) {
+  __shared__ float sx[HL_SMALL_K];
+  __shared__ float red[4][64];
+  const int t = blockIdx.x, h = blockIdx.y;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const TA* xr = in + (size_t)t * is + (size_t)h * ihs;
+  for (int k = threadIdx.x; k < K; k += blockDim.x) sx[k] = to_float(xr[k]);
+  __syncthreads();
+  const TA* Wh = W + (size_t)h * K * N;
+  const int per = (K + 3) >> 2;
+  const int kb = wave * per, ke = min(K, kb + per);
+  for (int n0 = 0; n0 < N; n0 += 64) {
+    const int n = min(n0 + lane, N - 1);
+    float acc = 0.f;
+    for (int k = kb; k < ke; k += 16) {
+      float wv[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) wv[u] = to_float(Wh[(size_t)min(k + u, ke - 1) * N + n]);
+#pragma unroll
+      for (int u = 0; u < 16; ++u) acc += (k + u < ke ? sx[min(k + u, HL_SMALL_K - 1)] : 0.f) * wv[u];
+    }
+    red[wave][lane] = acc;
+    __syncthreads();
+    if (wave == 0 && n0 + lane < N)
+      out[(size_t)t * os + (size_t)h * ohs + n0 + lane] =
+          from_float<TA>(((red[0][lane] + red[1][lane]) + red[2][lane]) + red[3][lane]);
+    __syncthreads();
+  }
+}
+
 extern "C" int sa_head_linear(const void* in, int is, int ihs, const void* W, void* out, int os, int ohs,
                               int act_dtype, int T, int H, int K, int N, hipStream_t stream) {
   if (T <= 0) return 0;
   if (H <= 0 || K <= 0 || N <= 0 || H > 65535 || (N + 255) / 256 > 65535) return SA_ERR_ARG;
+  if (T <= 64 && K <= HL_SMALL_K) {
+    dim3 grid(T, H), block(256);
+    if (act_dtype == SA_F32)
+      hipLaunchKernelGGL(head_linear_small_kernel<float>, grid, block, 0, stream, (const float*)in, is, ihs,
+                         (const float*)W, (float*)out, os, ohs, K, N);
+    else if (act_dtype == SA_BF16)
+      hipLaunchKernelGGL(head_linear_small_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)in, is, ihs,
+                         (const bf16_t*)W, (bf16_t*)out, os, ohs, K, N);
+    else return SA_ERR_UNSUPPORTED;
+    SA_LAUNCH_CHECK();
+    return 0;
+  }
   const int bx = N >= 256 ? 256 : ((N + 63) / 64) * 64;
   dim3 grid((T + HL_TT - 1) / HL_TT, H, (N + bx - 1) / bx), block(bx);
   if (act_dtype == SA_F32)

@@ -288,6 +288,22 @@ def test_experts_against_one_by_one(dtype, T, d, F):
             assert torch.allclose(yk[t * top + k].double(), want, atol=2e-4 if dtype == torch.float32 else 2e-2, rtol=1e-3)
 
 
+@pytest.mark.parametrize("T", [1, 9, 64, 65, 200])          # a workgroup per (token, head) up to 64 tokens, tiles of tokens above
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_per_head_products(dtype, T):
+    from serve_amd import ops
+    torch.manual_seed(T)
+    H, K, N, stride_in, stride_out = 5, 37, 70, 5 * 48, 5 * 80      # heads' inputs and outputs lie inside wider rows
+    x = torch.randn(T, stride_in, device="cuda").to(dtype)
+    w = (torch.randn(H, K, N, device="cuda") * 0.3).to(dtype)
+    out = torch.full((T, stride_out), 7.0, device="cuda").to(dtype)
+    ops.head_linear(x, stride_in, 48, w, out, stride_out, 80, T)
+    want = torch.einsum("thk,hkn->thn", x.view(T, H, 48)[:, :, :K].double(), w.double())
+    got = out.view(T, H, 80)
+    assert torch.allclose(got[:, :, :N].double(), want, atol=1e-4 if dtype == torch.float32 else 5e-2, rtol=1e-2)
+    assert (got[:, :, N:] == 7.0).all(), "a place behind a head's outputs was written"
+
+
 @pytest.mark.parametrize("longest", [1, 64])      # which shape of the recurrence kernel runs: single tokens, prompt portions
 @pytest.mark.parametrize("dk,dv,heads,kv_heads,taps", [(16, 24, 4, 2, 3), (72, 80, 2, 1, 4), (200, 8, 1, 1, 1), (33, 130, 3, 3, 2)])
 def test_delta_rule_kernels_in_two_steps(dk, dv, heads, kv_heads, taps, longest):

@@ -1,7 +1,7 @@
 // Paged attention in fp32 arithmetic: one wave per (token, query head) (below), and for prompt
 // portions of the float32 path a kernel that shares keys and values across 64 rows (further down).
 //
-// The first is the general form: any head_dim up to 256, any head counts, any page size, any mix of
+// The first is the general form: any head_dim up to 640, any head counts, any page size, any mix of
 // prompt portions and single tokens in one launch.  Formulas as in serve/kernels/attn_prefill.py:56-72,205 and attn_decode.py:99-111,236:
 // scores = q.k * scale, key j visible to the query at absolute position p iff j <= p (and
 // p - j < window when a window is set), online softmax (m, l, O), O / l at the end.  Query head
@@ -13,7 +13,7 @@
 // k pages [page, Hk, page_size, D]; v pages [page, Hk, D, page_size].
 #include "common.h"
 
-#define SA_MAX_D 256
+#define SA_MAX_D 640
 
 template <typename TA, typename TC>
 __global__ __launch_bounds__(64) void paged_attention_simple_kernel(

@@ -230,6 +230,9 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Te
                               c_int(page_size), c_int(1 if write else 0), _stream()), "rope_kv_write")
 
 
+SIMPLE_ATTENTION_MAX_HEAD_DIM = 640     # (SA_MAX_D of csrc/attention_simple.hip)
+
+
 def paged_attention_simple(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pages: torch.Tensor,
                            v_pages: torch.Tensor, block_table: torch.Tensor, cu_q: torch.Tensor,
                            ctx_len: torch.Tensor, seg_of_token: torch.Tensor, num_tokens: int,
@@ -242,7 +245,7 @@ def paged_attention_simple(q: torch.Tensor, q_row_stride: int, out: torch.Tensor
     P, Hk, page_size, D = k_pages.shape
     _check(v_pages.shape == (P, Hk, D, page_size), "v_pages must be [P, Hk, D, page_size]")
     _check(num_heads % Hk == 0, "query heads must be a multiple of KV heads")
-    _check(D <= 256, f"head_dim {D} is above this kernel's limit of 256")
+    _check(D <= SIMPLE_ATTENTION_MAX_HEAD_DIM, f"head_dim {D} is above this kernel's limit of {SIMPLE_ATTENTION_MAX_HEAD_DIM}")
     T = num_tokens
     _check(out.shape == (T, num_heads * D) and out.dtype == q.dtype, "attention output must be [T, Hq D]")
     _check(q.numel() >= (T - 1) * q_row_stride + num_heads * D if T else True, "q is too short")

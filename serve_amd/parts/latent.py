@@ -24,7 +24,7 @@ from .base import CacheTensor, LayerCache, ParamRequest, Part, Runtime, StepCost
 from .linear import linear
 from .standard import _prepare_products
 
-LATENT_MAX_ROW = 256        # the widest cache row the attention kernels take
+LATENT_MAX_ROW = ops.SIMPLE_ATTENTION_MAX_HEAD_DIM        # the widest cache row the attention kernels take
 
 
 class LatentAttention(Part):

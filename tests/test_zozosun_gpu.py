@@ -16,7 +16,7 @@ from tests import zozosun_models as zm
 pytestmark = pytest.mark.gpu
 
 DTYPES = ["float32", "bfloat16"]
-NAMES = ["ZA", "ZB", "ZD", "ZL"]
+NAMES = ["ZA", "ZB", "ZD", "ZL", "ZO"]
 
 
 def tokens_for(folder, dtype, n, seed, vocab):

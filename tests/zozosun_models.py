@@ -56,7 +56,15 @@ ZL = ZozosunConfig(vocab=150, width=80, eps=1e-5, layers=(
     L(_latent(2, 32, 32, 32, 64, 17, scale=0.125, base=500000.0), DenseMlpConfig(72)),
 ))
 
-MODELS = {"ZA": (ZA, 3), "ZB": (ZB, 4), "ZD": (ZD, 5), "ZL": (ZL, 6)}
+# sizes that no kernel's vector path takes: a width that is no multiple of 4, odd head sizes and widths of
+# experts, a cache row of 290 (above the tiled attention kernels), one tap more than the others
+ZO = ZozosunConfig(vocab=101, width=50, eps=1e-5, layers=(
+    L(_delta(3, 1, 10, 7, 5), MoeMlpConfig(3, 2, 9, 5)),
+    L(_latent(3, 6, 10, 5, 270, 11, scale=0.3), DenseMlpConfig(30)),
+    L(_latent(1, 5, 10, 9, 270, 4, scale=0.3, kv_from=1), None),
+))
+
+MODELS = {"ZA": (ZA, 3), "ZB": (ZB, 4), "ZD": (ZD, 5), "ZL": (ZL, 6), "ZO": (ZO, 7)}
 
 # queries and the keys' up-projections drawn wide: scores of order one, so that softmax picks keys and a
 # window that is one token off, a wrong rotation or a wrong head shows in the logits

@@ -9,7 +9,8 @@
 //   latent_kv_write   c = z[:R] / sqrt(mean(z[:R]^2) + eps) * w,  kr = rot(z[R:], position)  -> pages
 //   head_linear       out[t, h, :] = in[t, h, :] W[h]  (W [H, K, N]): the queries into the latent
 //                     space, and the latent outputs out of it
-//   latent_q_rot      the rotated part of every query head, and the padding of its row
+//                     (behind a head's outputs it can put the rotated part of the query and the row's padding,
+//                     so that the queries are one kernel)
 //
 // Rotation: dimension i of the rotated part is paired with i + dr/2; (u, v) -> (u cos a - v sin a,
 // v cos a + u sin a), a = position * inv_freq[i], in fp32.
@@ -89,10 +90,36 @@ extern "C" int sa_latent_kv_write(const void* z, int act_dtype, const float* w, 
 #define HL_TT 8
 #define HL_KC 128
 
+// What may follow a head's N outputs in its row of `out` (the queries of latent attention): the `rot` inputs that
+// lie behind the head's K inputs, rotated by the token's position, then zeros up to `tail` places.
+struct HeadTail {
+  const int* positions;      // nullptr: no tail
+  const float* inv_freq;     // [rot / 2]
+  int rot, tail;
+};
+
+template <typename TA>
+__device__ __forceinline__ void write_tail(const HeadTail& ht, const TA* __restrict__ src, TA* __restrict__ dst, int t,
+                                           int first, int step) {
+  const float pos = (float)ht.positions[t];
+  const int half = ht.rot / 2;
+  for (int i = first; i < ht.tail; i += step) {
+    float v = 0.f;
+    if (i < ht.rot) {
+      const int jf = i < half ? i : i - half;
+      float sn, cs;
+      sincos_for<TA>(pos * ht.inv_freq[jf], &sn, &cs);
+      const float a = to_float(src[jf]), b = to_float(src[jf + half]);
+      v = i < half ? a * cs - b * sn : b * cs + a * sn;
+    }
+    dst[i] = from_float<TA>(v);
+  }
+}
+
 template <typename TA>
 __global__ __launch_bounds__(256) void head_linear_kernel(const TA* __restrict__ in, int is, int ihs,
                                                           const TA* __restrict__ W, TA* __restrict__ out, int os,
-                                                          int ohs, int T, int K, int N) {
+                                                          int ohs, int T, int K, int N, HeadTail ht) {
   __shared__ float sin_[HL_TT][HL_KC];
   const int t0 = blockIdx.x * HL_TT;
   const int h = blockIdx.y;
@@ -122,6 +149,11 @@ __global__ __launch_bounds__(256) void head_linear_kernel(const TA* __restrict__
     for (int tt = 0; tt < HL_TT; ++tt)
       if (t0 + tt < T) out[(size_t)(t0 + tt) * os + (size_t)h * ohs + n] = from_float<TA>(acc[tt]);
   }
+  if (ht.positions && blockIdx.z == 0) {
+    for (int tt = 0; tt < HL_TT && t0 + tt < T; ++tt)
+      write_tail<TA>(ht, in + (size_t)(t0 + tt) * is + (size_t)h * ihs + K,
+                     out + (size_t)(t0 + tt) * os + (size_t)h * ohs + N, t0 + tt, threadIdx.x, blockDim.x);
+  }
 }
 
 // The same for few tokens (single decoded tokens): a workgroup per (token, head), the four waves cut K between
@@ -132,13 +164,14 @@ __global__ __launch_bounds__(256) void head_linear_kernel(const TA* __restrict__
 template <typename TA>
 __global__ __launch_bounds__(256) void head_linear_small_kernel(const TA* __restrict__ in, int is, int ihs,
                                                                 const TA* __restrict__ W, TA* __restrict__ out, int os,
-                                                                int ohs, int K, int N) {
+                                                                int ohs, int K, int N, HeadTail ht) {
   __shared__ float sx[HL_SMALL_K];
   __shared__ float red[4][64];
   const int t = blockIdx.x, h = blockIdx.y;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const TA* xr = in + (size_t)t * is + (size_t)h * ihs;
   for (int k = threadIdx.x; k < K; k += blockDim.x) sx[k] = to_float(xr[k]);
+  if (ht.positions) write_tail<TA>(ht, xr + K, out + (size_t)t * os + (size_t)h * ohs + N, t, threadIdx.x, blockDim.x);
   __syncthreads();
   const TA* Wh = W + (size_t)h * K * N;
   const int per = (K + 3) >> 2;
@@ -163,17 +196,20 @@ __global__ __launch_bounds__(256) void head_linear_small_kernel(const TA* __rest
 }
 
 extern "C" int sa_head_linear(const void* in, int is, int ihs, const void* W, void* out, int os, int ohs,
-                              int act_dtype, int T, int H, int K, int N, hipStream_t stream) {
+                              int act_dtype, int T, int H, int K, int N, const int* positions, const float* inv_freq,
+                              int rot, int tail, hipStream_t stream) {
   if (T <= 0) return 0;
   if (H <= 0 || K <= 0 || N <= 0 || H > 65535 || (N + 255) / 256 > 65535) return SA_ERR_ARG;
+  if (positions && ((!inv_freq && rot > 0) || rot < 0 || (rot & 1) || tail < rot)) return SA_ERR_ARG;
+  HeadTail ht = {positions, inv_freq, rot, tail};
   if (T <= 64 && K <= HL_SMALL_K) {
     dim3 grid(T, H), block(256);
     if (act_dtype == SA_F32)
       hipLaunchKernelGGL(head_linear_small_kernel<float>, grid, block, 0, stream, (const float*)in, is, ihs,
-                         (const float*)W, (float*)out, os, ohs, K, N);
+                         (const float*)W, (float*)out, os, ohs, K, N, ht);
     else if (act_dtype == SA_BF16)
       hipLaunchKernelGGL(head_linear_small_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)in, is, ihs,
-                         (const bf16_t*)W, (bf16_t*)out, os, ohs, K, N);
+                         (const bf16_t*)W, (bf16_t*)out, os, ohs, K, N, ht);
     else return SA_ERR_UNSUPPORTED;
     SA_LAUNCH_CHECK();
     return 0;
@@ -182,53 +218,10 @@ extern "C" int sa_head_linear(const void* in, int is, int ihs, const void* W, vo
   dim3 grid((T + HL_TT - 1) / HL_TT, H, (N + bx - 1) / bx), block(bx);
   if (act_dtype == SA_F32)
     hipLaunchKernelGGL(head_linear_kernel<float>, grid, block, 0, stream, (const float*)in, is, ihs, (const float*)W,
-                       (float*)out, os, ohs, T, K, N);
+                       (float*)out, os, ohs, T, K, N, ht);
   else if (act_dtype == SA_BF16)
     hipLaunchKernelGGL(head_linear_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)in, is, ihs,
-                       (const bf16_t*)W, (bf16_t*)out, os, ohs, T, K, N);
-  else return SA_ERR_UNSUPPORTED;
-  SA_LAUNCH_CHECK();
-  return 0;
-}
-
-// ---------------------------------------------------------------------------------------------
-// qf[t, h, R + i] = rot(q[t, h, dn + i]) for i < dr, and qf[t, h, R + dr ..] = 0.
-// q [T, H (dn + dr)], qf [T, H Dp].  grid (T, H).
-// ---------------------------------------------------------------------------------------------
-template <typename TA>
-__global__ __launch_bounds__(64) void latent_q_rot_kernel(const TA* __restrict__ q, const int* __restrict__ positions,
-                                                          const float* __restrict__ inv_freq, TA* __restrict__ qf,
-                                                          int H, int dn, int dr, int R, int Dp) {
-  const int t = blockIdx.x, h = blockIdx.y;
-  const TA* qr = q + ((size_t)t * H + h) * (dn + dr) + dn;
-  TA* dst = qf + ((size_t)t * H + h) * Dp + R;
-  const float pos = (float)positions[t];
-  const int half = dr / 2;
-  for (int i = threadIdx.x; i < Dp - R; i += blockDim.x) {
-    float v = 0.f;
-    if (i < dr) {
-      const int jf = i < half ? i : i - half;
-      float sn, cs;
-      sincos_for<TA>(pos * inv_freq[jf], &sn, &cs);
-      const float a = to_float(qr[jf]), b = to_float(qr[jf + half]);
-      v = i < half ? a * cs - b * sn : b * cs + a * sn;
-    }
-    dst[i] = from_float<TA>(v);
-  }
-}
-
-extern "C" int sa_latent_q_rot(const void* q, int act_dtype, const int* positions, const float* inv_freq, void* qf,
-                               int T, int H, int dn, int dr, int R, int Dp, hipStream_t stream) {
-  if (T <= 0) return 0;
-  if (H <= 0 || H > 65535 || dn < 0 || dr < 0 || (dr & 1) || R <= 0 || Dp < R + dr) return SA_ERR_ARG;
-  if (Dp == R) return 0;
-  dim3 grid(T, H), block(64);
-  if (act_dtype == SA_F32)
-    hipLaunchKernelGGL(latent_q_rot_kernel<float>, grid, block, 0, stream, (const float*)q, positions, inv_freq,
-                       (float*)qf, H, dn, dr, R, Dp);
-  else if (act_dtype == SA_BF16)
-    hipLaunchKernelGGL(latent_q_rot_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)q, positions, inv_freq,
-                       (bf16_t*)qf, H, dn, dr, R, Dp);
+                       (const bf16_t*)W, (bf16_t*)out, os, ohs, T, K, N, ht);
   else return SA_ERR_UNSUPPORTED;
   SA_LAUNCH_CHECK();
   return 0;

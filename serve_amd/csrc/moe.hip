@@ -23,12 +23,19 @@
 // ---------------------------------------------------------------------------------------------
 // route: a wave per token.  Ties go to the lower index.
 // ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ void route_token(const float* __restrict__ z, int* __restrict__ ids, float* __restrict__ wts,
+                                            int E, int top, int lane);
+
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int ldz, int* __restrict__ ids,
                                                         float* __restrict__ wts, int T, int E, int top) {
   const int t = blockIdx.x * (blockDim.x / SA_WAVE) + threadIdx.x / SA_WAVE;
   if (t >= T) return;
-  const int lane = threadIdx.x & (SA_WAVE - 1);
-  const float* z = logits + (size_t)t * ldz;
+  route_token(logits + (size_t)t * ldz, ids + (size_t)t * top, wts + (size_t)t * top, E, top,
+              threadIdx.x & (SA_WAVE - 1));
+}
+
+__device__ __forceinline__ void route_token(const float* __restrict__ z, int* __restrict__ ids, float* __restrict__ wts,
+                                            int E, int top, int lane) {
   float prev_v = INFINITY;
   int prev_i = -1;
   float first = 0.f, sum = 0.f;
@@ -51,14 +58,14 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
     const float p = expf(bv - first);
     sum += p;
     if (lane == 0) {
-      ids[(size_t)t * top + k] = bi;
-      wts[(size_t)t * top + k] = p;
+      ids[k] = bi;
+      wts[k] = p;
     }
     prev_v = bv;
     prev_i = bi;
   }
   if (lane == 0)
-    for (int k = 0; k < top; ++k) wts[(size_t)t * top + k] /= sum;
+    for (int k = 0; k < top; ++k) wts[k] /= sum;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -66,11 +73,20 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
 // takes the next free row of its expert (the order inside an expert does not matter: a row's sums
 // do not depend on its place).
 // ---------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__ ids, int n, int E, int tile_rows,
+__global__ __launch_bounds__(1024) void moe_group_kernel(const int* ids, int n, int E, int tile_rows,
                                                          int* __restrict__ offsets, int* __restrict__ cursor,
                                                          int* __restrict__ perm, int* __restrict__ tile_expert,
-                                                         int* __restrict__ tile_row0, int* __restrict__ num_tiles) {
+                                                         int* __restrict__ tile_row0, int* __restrict__ num_tiles,
+                                                         const float* __restrict__ logits, int ldz, int* ids_out,
+                                                         float* __restrict__ wts, int top) {
   for (int e = threadIdx.x; e < E; e += blockDim.x) cursor[e] = 0;
+  if (logits) {
+    // a step of few tokens: the routing is done here, a wave a token in turn, and saves a kernel
+    const int waves = blockDim.x / SA_WAVE, T = n / top;
+    for (int t = threadIdx.x / SA_WAVE; t < T; t += waves)
+      route_token(logits + (size_t)t * ldz, ids_out + (size_t)t * top, wts + (size_t)t * top, E, top,
+                  threadIdx.x & (SA_WAVE - 1));
+  }
   __syncthreads();
   for (int i = threadIdx.x; i < n; i += blockDim.x) atomicAdd(&cursor[ids[i]], 1);
   __syncthreads();
@@ -404,9 +420,14 @@ extern "C" int sa_moe_route(const float* logits, int ldz, int* ids, float* wts, 
 // MOE_SMALL_ROWS rows (T top) in tiles of 16 with K cut over the waves, more in tiles of 64.
 #define MOE_SMALL_ROWS 1024
 
-extern "C" int sa_moe_experts(const void* h, int act_dtype, const int* ids, const void* Wg, const void* Wu,
+// logits != nullptr (and T <= MOE_ROUTE_INSIDE): ids and wts are made here from the router's logits fp32 [T, ldz]
+#define MOE_ROUTE_INSIDE 16
+
+extern "C" int sa_moe_route_inside_limit() { return MOE_ROUTE_INSIDE; }
+
+extern "C" int sa_moe_experts(const void* h, int act_dtype, int* ids, const void* Wg, const void* Wu,
                               const void* Wd, int* ints, void* act, float* yk, int T, int top, int E, int d, int F,
-                              hipStream_t stream) {
+                              const float* logits, int ldz, float* wts, hipStream_t stream) {
   if (T <= 0) return 0;
   const long long n = (long long)T * top;
   if (E <= 0 || top <= 0 || d <= 0 || F <= 0 || n > 0x3fffffffLL) return SA_ERR_ARG;
@@ -421,8 +442,9 @@ extern "C" int sa_moe_experts(const void* h, int act_dtype, const int* ids, cons
   const bool small = n <= MOE_SMALL_ROWS;
   const int tile_rows = mfma ? (small ? 16 : 64) : MOE_TM;
   const int tiles = (int)((n + tile_rows - 1) / tile_rows) + E;
+  if (logits && (T > MOE_ROUTE_INSIDE || !wts || ldz < E || top > E)) return SA_ERR_ARG;
   hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), 0, stream, ids, (int)n, E, tile_rows, offsets, cursor, perm,
-                     tile_expert, tile_row0, num_tiles);
+                     tile_expert, tile_row0, num_tiles, logits, ldz, ids, wts, top);
   SA_LAUNCH_CHECK();
   dim3 block(256);
   if (mfma) {
@@ -431,17 +453,17 @@ extern "C" int sa_moe_experts(const void* h, int act_dtype, const int* ids, cons
     const int per = small ? 16 : 128;          // weight rows a workgroup owns
     dim3 g1(tiles, (F + per - 1) / per), g2(tiles, (d + per - 1) / per);
     if (g1.y > 65535 || g2.y > 65535) return SA_ERR_ARG;
-#define GO(MT, KS, WR)                                                                                                   \
+#define GO(MT, KS, WR, KU)                                                                                                   \
   do {                                                                                                                 \
-    hipLaunchKernelGGL((moe_mfma_kernel<MT, KS, true, WR>), g1, block, 0, stream, (const bf16_t*)h, (const bf16_t*)Wg,     \
+    hipLaunchKernelGGL((moe_mfma_kernel<MT, KS, true, WR, KU>), g1, block, 0, stream, (const bf16_t*)h, (const bf16_t*)Wg,     \
                        (const bf16_t*)Wu, offsets, perm, tile_expert, tile_row0, num_tiles, (bf16_t*)act, nullptr,     \
                        top, F, d);                                                                                     \
     SA_LAUNCH_CHECK();                                                                                                 \
-    hipLaunchKernelGGL((moe_mfma_kernel<MT, KS, false, WR>), g2, block, 0, stream, (const bf16_t*)act, (const bf16_t*)Wd,  \
+    hipLaunchKernelGGL((moe_mfma_kernel<MT, KS, false, WR, KU>), g2, block, 0, stream, (const bf16_t*)act, (const bf16_t*)Wd,  \
                        nullptr, offsets, perm, tile_expert, tile_row0, num_tiles, nullptr, yk, top, d, F);             \
   } while (0)
-    if (small) GO(1, 4, 1);
-    else GO(4, 1, 2);
+    if (small) GO(1, 4, 1, 2);
+    else GO(4, 1, 2, 2);
 #undef GO
     SA_LAUNCH_CHECK();
     return 0;

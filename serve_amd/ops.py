@@ -498,37 +498,32 @@ def latent_kv_write(z: torch.Tensor, norm_w: torch.Tensor, positions: torch.Tens
 
 
 def head_linear(x: torch.Tensor, in_stride: int, in_head_stride: int, w: torch.Tensor, out: torch.Tensor,
-                out_stride: int, out_head_stride: int, T: int) -> torch.Tensor:
+                out_stride: int, out_head_stride: int, T: int, positions: Optional[torch.Tensor] = None,
+                inv_freq: Optional[torch.Tensor] = None, rot: int = 0, tail: int = 0) -> torch.Tensor:
     """out[t, h, :N] = x[t, h, :K] @ w[h] for w [H, K, N]: head h's K inputs of token t start at element
-    t * in_stride + h * in_head_stride of x, its N outputs at t * out_stride + h * out_head_stride of out."""
-    _dev(x, w, out)
+    t * in_stride + h * in_head_stride of x, its N outputs at t * out_stride + h * out_head_stride of out.
+    With `positions`: behind the N outputs come the `rot` inputs that lie behind the head's K inputs, rotated by
+    the token's position (dimension i with i + rot / 2, angles positions[t] * inv_freq[i]), then zeros up to
+    `tail` places in all."""
+    _dev(x, w, out, positions, inv_freq)
     _check(w.dim() == 3 and x.dtype == w.dtype == out.dtype, "head_linear: w must be [H, K, N], one dtype throughout")
     H, K, N = w.shape
     if T:
         _check(x.numel() >= (T - 1) * in_stride + (H - 1) * in_head_stride + K, "head_linear: input too short")
-        _check(out.numel() >= (T - 1) * out_stride + (H - 1) * out_head_stride + N, "head_linear: output too short")
+        _check(out.numel() >= (T - 1) * out_stride + (H - 1) * out_head_stride + N + tail, "head_linear: output too short")
+    if positions is not None:
+        _i32(positions, T, "positions")
+        _check(rot % 2 == 0 and 0 <= rot <= tail and in_head_stride >= K + rot and out_head_stride >= N + tail,
+               "head_linear: the rotated inputs lie behind a head's K inputs, the tail behind its N outputs")
+        _f32vec(inv_freq, rot // 2, "inv_freq")
+        if T:
+            _check(x.numel() >= (T - 1) * in_stride + (H - 1) * in_head_stride + K + rot, "head_linear: input too short")
     lib = load_library("latent")
     _ret(lib.sa_head_linear(_ptr(x), c_int(in_stride), c_int(in_head_stride), _ptr(w), _ptr(out), c_int(out_stride),
-                            c_int(out_head_stride), c_int(_code(x)), c_int(T), c_int(H), c_int(K), c_int(N), _stream()),
+                            c_int(out_head_stride), c_int(_code(x)), c_int(T), c_int(H), c_int(K), c_int(N),
+                            _ptr(positions), _ptr(inv_freq), c_int(rot), c_int(tail), _stream()),
          "head_linear")
     return out
-
-
-def latent_q_rot(q: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor, qf: torch.Tensor, heads: int,
-                 dim: int, rot_dim: int, rank: int) -> None:
-    """The rotated part of every query head into its place behind the `rank` latent dims of the head's
-    row of qf [T, H Dp], and zeros behind it.  q [T, H (dim + rot_dim)]."""
-    _dev(q, positions, inv_freq, qf)
-    T = q.shape[0]
-    _check(q.shape == (T, heads * (dim + rot_dim)) and qf.dim() == 2 and qf.shape[0] == T and qf.shape[1] % heads == 0
-           and qf.dtype == q.dtype, "latent_q_rot: q [T, H (dim + rot_dim)], qf [T, H Dp]")
-    Dp = qf.shape[1] // heads
-    _check(Dp >= rank + rot_dim, "latent_q_rot: rows of qf are too short")
-    _f32vec(inv_freq, rot_dim // 2, "inv_freq")
-    _i32(positions, T, "positions")
-    lib = load_library("latent")
-    _ret(lib.sa_latent_q_rot(_ptr(q), c_int(_code(q)), _ptr(positions), _ptr(inv_freq), _ptr(qf), c_int(T),
-                             c_int(heads), c_int(dim), c_int(rot_dim), c_int(rank), c_int(Dp), _stream()), "latent_q_rot")
 
 
 # ---------------------------------------------------------------------------------------------
@@ -549,11 +544,16 @@ def moe_route(logits: torch.Tensor, experts: int, top: int, ids: torch.Tensor, w
                           c_int(top), _stream()), "moe_route")
 
 
+MOE_ROUTE_INSIDE = 16      # up to this many tokens the experts' call does the routing itself (one kernel less)
+
+
 def moe_experts(h: torch.Tensor, ids: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor,
-                yk: torch.Tensor) -> torch.Tensor:
+                yk: torch.Tensor, logits: Optional[torch.Tensor] = None,
+                weights: Optional[torch.Tensor] = None) -> torch.Tensor:
     """yk[t * top + k] = expert ids[t, k] applied to h[t]: down(silu(gate h) * up h), fp32 [T top, d].
-    w_gate, w_up [E, F, d], w_down [E, d, F] in h's dtype."""
-    _dev(h, ids, w_gate, w_up, w_down, yk)
+    w_gate, w_up [E, F, d], w_down [E, d, F] in h's dtype.  With `logits` (fp32 [T, >= E], at most
+    MOE_ROUTE_INSIDE tokens) `ids` and `weights` are made here as `moe_route` makes them."""
+    _dev(h, ids, w_gate, w_up, w_down, yk, logits, weights)
     T, d = h.shape
     top = ids.shape[1]
     E, F, d2 = w_gate.shape
@@ -566,9 +566,16 @@ def moe_experts(h: torch.Tensor, ids: torch.Tensor, w_gate: torch.Tensor, w_up: 
     tiles = int(lib.sa_moe_max_tiles(c_int(n), c_int(E)))
     ints = torch.empty(2 * E + 1 + n + 2 * tiles + 1, dtype=torch.int32, device=h.device)
     act = torch.empty((n, F), dtype=h.dtype, device=h.device)
+    ldz = 0
+    if logits is not None:
+        _check(T <= MOE_ROUTE_INSIDE and logits.dtype == torch.float32 and logits.dim() == 2 and logits.shape[0] == T
+               and logits.shape[1] >= E and 0 < top <= E, "moe_experts: logits fp32 [T, >= E] of at most "
+               f"{MOE_ROUTE_INSIDE} tokens")
+        _check(weights is not None and weights.dtype == torch.float32 and weights.shape == (T, top), "weights fp32 [T, top]")
+        ldz = logits.shape[1]
     _ret(lib.sa_moe_experts(_ptr(h), c_int(_code(h)), _ptr(ids), _ptr(w_gate), _ptr(w_up), _ptr(w_down), _ptr(ints),
-                            _ptr(act), _ptr(yk), c_int(T), c_int(top), c_int(E), c_int(d), c_int(F), _stream()),
-         "moe_experts")
+                            _ptr(act), _ptr(yk), c_int(T), c_int(top), c_int(E), c_int(d), c_int(F), _ptr(logits),
+                            c_int(ldz), _ptr(weights), _stream()), "moe_experts")
     return yk
 
 

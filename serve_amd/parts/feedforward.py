@@ -103,9 +103,12 @@ class RoutedExperts(Part):
         logits = linear(h, self.w_router, out_dtype=torch.float32)
         ids = torch.empty((T, self.top), dtype=torch.int32, device=dev)
         weights = torch.empty((T, self.top), dtype=torch.float32, device=dev)
-        ops.moe_route(logits, self.experts, self.top, ids, weights)
         yk = torch.empty((T * self.top, d), dtype=torch.float32, device=dev)
-        ops.moe_experts(h, ids, self.w_gate, self.w_up, self.w_down, yk)
+        if T <= ops.MOE_ROUTE_INSIDE:
+            ops.moe_experts(h, ids, self.w_gate, self.w_up, self.w_down, yk, logits, weights)   # routes, too
+        else:
+            ops.moe_route(logits, self.experts, self.top, ids, weights)
+            ops.moe_experts(h, ids, self.w_gate, self.w_up, self.w_down, yk)
         shared = self.shared.forward(h, ctx) if self.shared is not None else None
         y = torch.empty((T, d), dtype=torch.float32, device=dev)
         return ops.moe_combine(yk, weights, shared, logits if self.shared_gate else None, self.experts, y)

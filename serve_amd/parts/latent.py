@@ -112,8 +112,9 @@ class LatentAttention(Part):
                                     self.eps, R, self.rot_dim)
             q = linear(h, self.wq)
             qf = self.rt.empty((T, H * D))
-            ops.head_linear(q, q.shape[1], self.dim + self.rot_dim, self.w_uk, qf, H * D, D, T)
-            ops.latent_q_rot(q, ctx.positions, self.inv_freq, qf, H, self.dim, self.rot_dim, R)
+            # the queries into the latent space, their rotated parts behind them, zeros up to the row's end
+            ops.head_linear(q, q.shape[1], self.dim + self.rot_dim, self.w_uk, qf, H * D, D, T, ctx.positions,
+                            self.inv_freq, self.rot_dim, D - R)
         attn = self.rt.empty((T, H * D))
         with trace.span("attention"):
             ops.paged_attention(qf, H * D, attn, k_pages, v_pages, grp.block_table, ctx, H, self.scale, self.window)

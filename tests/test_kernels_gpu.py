@@ -829,10 +829,10 @@ def test_kernels_refuse_what_they_do_not_take():
         ops.gemm_nt(a.cpu(), w.cpu(), out.cpu())
     k_pages = torch.zeros((2, 1, 8, 144), dtype=torch.bfloat16, device=DEV)
     assert not ops.mfma_attention_available(rnd((1, 144), torch.bfloat16, 1), k_pages, 144)   # head size 144
-    with pytest.raises(ops.KernelError, match="256"):
-        big = torch.zeros((2, 1, 8, 272), dtype=torch.float32, device=DEV)
-        ops.paged_attention_simple(rnd((1, 272), torch.float32, 1), 272, torch.empty((1, 272), device=DEV), big,
-                                   torch.zeros((2, 1, 272, 8), device=DEV),
+    with pytest.raises(ops.KernelError, match="640"):
+        big = torch.zeros((2, 1, 8, 656), dtype=torch.float32, device=DEV)
+        ops.paged_attention_simple(rnd((1, 656), torch.float32, 1), 656, torch.empty((1, 656), device=DEV), big,
+                                   torch.zeros((2, 1, 656, 8), device=DEV),
                                    torch.zeros((1, 1), dtype=torch.int32, device=DEV),
                                    torch.tensor([0, 1], dtype=torch.int32, device=DEV),
                                    torch.tensor([1], dtype=torch.int32, device=DEV),

@@ -264,6 +264,24 @@ def test_route_picks_the_largest_and_weights_them_among_themselves(experts, top)
     assert torch.allclose(w.double(), torch.softmax(vals, -1), atol=1e-6)
 
 
+def test_experts_route_by_themselves_for_few_tokens():
+    from serve_amd import ops
+    torch.manual_seed(9)
+    T, d, F, E, top = 13, 64, 32, 9, 3
+    h = torch.randn(T, d, device="cuda").bfloat16()
+    wg, wu = (torch.randn(E, F, d, device="cuda") * 0.2).bfloat16(), (torch.randn(E, F, d, device="cuda") * 0.2).bfloat16()
+    wd = (torch.randn(E, d, F, device="cuda") * 0.2).bfloat16()
+    logits = torch.randn(T, E + 1, device="cuda")
+    ids_a, w_a = torch.empty(T, top, dtype=torch.int32, device="cuda"), torch.empty(T, top, device="cuda")
+    ops.moe_route(logits, E, top, ids_a, w_a)
+    yk_a = torch.empty(T * top, d, device="cuda")
+    ops.moe_experts(h, ids_a, wg, wu, wd, yk_a)
+    ids_b, w_b = torch.full((T, top), -1, dtype=torch.int32, device="cuda"), torch.zeros(T, top, device="cuda")
+    yk_b = torch.empty(T * top, d, device="cuda")
+    ops.moe_experts(h, ids_b, wg, wu, wd, yk_b, logits, w_b)
+    assert torch.equal(ids_a, ids_b) and torch.equal(w_a, w_b) and torch.equal(yk_a, yk_b)
+
+
 @pytest.mark.parametrize("T,d,F", [(45, 72, 40), (45, 75, 42), (400, 64, 48)])   # few rows; sizes the matrix cores do not take; many rows
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_experts_against_one_by_one(dtype, T, d, F):
@@ -300,8 +318,20 @@ def test_per_head_products(dtype, T):
     ops.head_linear(x, stride_in, 48, w, out, stride_out, 80, T)
     want = torch.einsum("thk,hkn->thn", x.view(T, H, 48)[:, :, :K].double(), w.double())
     got = out.view(T, H, 80)
-    assert torch.allclose(got[:, :, :N].double(), want, atol=1e-4 if dtype == torch.float32 else 5e-2, rtol=1e-2)
+    tol = dict(atol=1e-4 if dtype == torch.float32 else 5e-2, rtol=1e-2)
+    assert torch.allclose(got[:, :, :N].double(), want, **tol)
     assert (got[:, :, N:] == 7.0).all(), "a place behind a head's outputs was written"
+    # with a tail: the 6 inputs behind the K are rotated by position and put behind the N outputs, then 2 zeros
+    from tests.plain import zozosun_plain as zp
+    positions = torch.arange(3, 3 + T, dtype=torch.int32, device="cuda")
+    base = 50.0
+    inv_freq = torch.tensor([base ** (-2.0 * i / 6) for i in range(3)], dtype=torch.float32, device="cuda")
+    ops.head_linear(x, stride_in, 48, w, out, stride_out, 80, T, positions, inv_freq, 6, 8)
+    got = out.view(T, H, 80)
+    assert torch.allclose(got[:, :, :N].double(), want, **tol)
+    turned = zp.rotate(x.view(T, H, 48)[:, :, K: K + 6].double().cpu(), positions.cpu().long(), base)
+    assert torch.allclose(got[:, :, N: N + 6].double().cpu(), turned, **tol)
+    assert (got[:, :, N + 6: N + 8] == 0).all() and (got[:, :, N + 8:] == 7.0).all()
 
 
 @pytest.mark.parametrize("longest", [1, 64])      # which shape of the recurrence kernel runs: single tokens, prompt portions

@@ -53,7 +53,7 @@ ZD = ZozosunConfig(vocab=128, width=48, eps=1e-5, layers=(
 # latent attention alone, more heads than a matrix-core tile has rows, one layer that sees every key
 ZL = ZozosunConfig(vocab=150, width=80, eps=1e-5, layers=(
     L(_latent(20, 8, 4, 8, 28, None, scale=0.35), None),
-    L(_latent(2, 32, 32, 32, 64, 17, scale=0.125, base=500000.0), DenseMlpConfig(72)),
+    L(_latent(2, 24, 16, 40, 56, 17, scale=0.2, base=300000.0), DenseMlpConfig(72)),
 ))
 
 # sizes that no kernel's vector path takes: a width that is no multiple of 4, odd head sizes and widths of

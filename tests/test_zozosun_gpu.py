@@ -386,3 +386,52 @@ def test_delta_rule_kernels_in_two_steps(dk, dv, heads, kv_heads, taps, longest)
         g_ = torch.cat(got[r]).double()
         assert torch.allclose(g_, want[r], atol=3e-4, rtol=1e-3), f"request {r}: max diff {(g_ - want[r]).abs().max().item():.3g}"
     assert state[1].abs().max().item() == 0.0, "a slot that no segment named was written"
+
+
+# ---------------------------------------------------------------------------------------------
+# the trace runner as a user runs it
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_traces_through_the_program(tmp_path, dtype):
+    """`bin/trace_run` as a child process on a model folder: whole prompts, prompt then single tokens, portions, and
+    a mix of four live requests (the program has four state slots, and pages for 256 tokens), against the plain model."""
+    import json
+    import os
+    import subprocess
+    import numpy as np
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    name = "ZA"
+    folder = zm.make_folder(tmp_path, name, sharp=True)
+    vocab = zm.MODELS[name][0].vocab
+    reqs, steps = {}, []
+
+    def feed(key, n, portions, seed):
+        reqs[key] = tokens_for(folder, dtype, n, seed, vocab)
+        at = 0
+        for j, m in enumerate(portions):
+            steps.append(([(key, reqs[key][at: at + m])], [key] if j == len(portions) - 1 else []))
+            at += m
+        assert at == n
+    feed("whole", 50, [50], 1)
+    feed("tail", 70, [30] + [1] * 40, 2)
+    feed("cut", 61, [7, 2, 16, 3, 2, 9, 2, 11, 5, 4], 3)
+    mixed = {f"m{i}": tokens_for(folder, dtype, n, 40 + i, vocab) for i, n in enumerate([23, 41, 9, 30, 17, 2, 36, 12, 40])}
+    reqs.update(mixed)
+    steps.extend(mixed_trace(random.Random(5), mixed))
+    lines = [json.dumps({"step": i, "entries": [{"id": k, "tokens": t, "want": list(range(len(t)))} for k, t in entries],
+                         "end": ended}) for i, (entries, ended) in enumerate(steps)]
+    out = tmp_path / "out"
+    proc = subprocess.run([os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", dtype, "--out", str(out),
+                           "--max-tokens", "256"], input="\n".join(lines) + "\n", capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(len(steps))]
+    rows = {k: [] for k in reqs}
+    for i, (entries, _) in enumerate(steps):
+        arr = torch.from_numpy(np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(sum(len(t) for _, t in entries), vocab))
+        at = 0
+        for k, t in entries:
+            rows[k].append(arr[at: at + len(t)])
+            at += len(t)
+    assert sum(len(t) for t in reqs.values()) > 256          # pages went from request to request
+    pairs = [zm.kept_rows(torch.cat(rows[k]), folder, t, dtype, f"trace request {k}") for k, t in reqs.items()]
+    zm.assert_close_but_few(torch.cat([g for g, _ in pairs]), torch.cat([w for _, w in pairs]), dtype, "all requests of the traces")

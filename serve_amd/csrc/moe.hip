@@ -448,9 +448,10 @@ extern "C" int sa_moe_experts(const void* h, int act_dtype, int* ids, const void
   SA_LAUNCH_CHECK();
   dim3 block(256);
   if (mfma) {
-    // (tiles of 64 rows: a wave owns two groups of 16 weight rows per matrix, 128 a workgroup: 608 us against 874
-    // with one group, for 2,048 tokens, 32 experts of width 1,024, top 4, model width 2,048)
-    const int per = small ? 16 : 128;          // weight rows a workgroup owns
+    // (tiles of 64 rows: a wave owns four groups of 16 weight rows per matrix, 256 a workgroup: 542 us against 604
+    // with two groups and 874 with one, for 2,048 tokens, 32 experts of width 1,024, top 4, model width 2,048;
+    // tiles of 128 rows were no faster)
+    const int per = small ? 16 : 256;          // weight rows a workgroup owns
     dim3 g1(tiles, (F + per - 1) / per), g2(tiles, (d + per - 1) / per);
     if (g1.y > 65535 || g2.y > 65535) return SA_ERR_ARG;
 #define GO(MT, KS, WR, KU)                                                                                                   \
@@ -463,7 +464,7 @@ extern "C" int sa_moe_experts(const void* h, int act_dtype, int* ids, const void
                        nullptr, offsets, perm, tile_expert, tile_row0, num_tiles, nullptr, yk, top, d, F);             \
   } while (0)
     if (small) GO(1, 4, 1, 2);
-    else GO(4, 1, 2, 2);
+    else GO(4, 1, 4, 2);
 #undef GO
     SA_LAUNCH_CHECK();
     return 0;

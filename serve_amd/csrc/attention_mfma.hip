@@ -84,7 +84,7 @@ __device__ __forceinline__ void attention_tile(
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ block_table, int max_pages, const int* __restrict__ ctx_len, int Hq, int Hk,
     int page_size, int page_shift, float scale_log2e, int window, int num_splits,
-    float* __restrict__ part_o, float* __restrict__ part_ml) {
+    float* __restrict__ part_o, float* __restrict__ part_ml, const float* __restrict__ sinks) {
   constexpr int NT = 1;                                     // column tiles of 16 rows per wave
   const int lane = threadIdx.x & 63;
   const int g = lane >> 4;
@@ -381,6 +381,8 @@ __device__ __forceinline__ void attention_tile(
     lt += __shfl_xor(lt, 32, 64);
     if (!rvalid[n]) continue;
     if (num_splits == 1) {
+      // (a sink: one more term of the denominator, exp(sink) against scores that are kept as powers of two)
+      if (sinks) lt += __builtin_amdgcn_exp2f(fmaf(sinks[head[n]], 1.4426950408889634f, -m[n]));
       const float inv = 1.f / lt;
       bf16_t* op = out + ((size_t)tok[n] * Hq + head[n]) * HD;
 #pragma unroll
@@ -412,7 +414,8 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ block_table, int max_pages, const int* __restrict__ cu_q,
     const int* __restrict__ ctx_len, int Hq, int Hk, int page_size, int page_shift, float scale_log2e,
-    int window, int num_splits, float* __restrict__ part_o, float* __restrict__ part_ml) {
+    int window, int num_splits, float* __restrict__ part_o, float* __restrict__ part_ml,
+    const float* __restrict__ sinks) {
   const int w = blockIdx.x * 4 + (threadIdx.x >> 6);
   const int hk = blockIdx.y;
   const int seg = blockIdx.z / num_splits;
@@ -420,7 +423,7 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   const int q_begin = cu_q[seg];
   const int q_len = cu_q[seg + 1] - q_begin;
   attention_tile<PM>(w, seg, hk, sp, q_begin, q_len, q, q_stride, out, k_pages, v_pages, block_table, max_pages,
-                     ctx_len, Hq, Hk, page_size, page_shift, scale_log2e, window, num_splits, part_o, part_ml);
+                     ctx_len, Hq, Hk, page_size, page_shift, scale_log2e, window, num_splits, part_o, part_ml, sinks);
 }
 
 // The same for short contexts: the WS waves of a workgroup take the WS parts of the key range of one
@@ -435,7 +438,7 @@ __global__ __launch_bounds__(64 * WG_SPLITS) void paged_attention_mfma_wg_kernel
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ block_table, int max_pages, const int* __restrict__ cu_q,
     const int* __restrict__ ctx_len, int Hq, int Hk, int page_size, int page_shift, float scale_log2e,
-    int window) {
+    int window, const float* __restrict__ sinks) {
   __shared__ float part_o[WG_SPLITS * 16 * HD];
   __shared__ float part_ml[WG_SPLITS * 16 * 2];
   const int wave = threadIdx.x >> 6;
@@ -445,7 +448,7 @@ __global__ __launch_bounds__(64 * WG_SPLITS) void paged_attention_mfma_wg_kernel
   const int q_len = cu_q[seg + 1] - q_begin;
   attention_tile<PM, true>(0, seg, hk, wave, q_begin, q_len, q, q_stride, out, k_pages, v_pages, block_table,
                            max_pages, ctx_len, Hq, Hk, page_size, page_shift, scale_log2e, window, WG_SPLITS,
-                           part_o, part_ml);
+                           part_o, part_ml, nullptr);
   __syncthreads();
   if (wave != 0) return;
   const int lane = threadIdx.x & 63;
@@ -476,8 +479,9 @@ __global__ __launch_bounds__(64 * WG_SPLITS) void paged_attention_mfma_wg_kernel
       o[dt][3] += p.w * w;
     }
   }
-  const float inv = 1.f / L;
   const int j = c / G;
+  if (sinks) L += __builtin_amdgcn_exp2f(fmaf(sinks[hk * G + (c - j * G)], 1.4426950408889634f, -M));
+  const float inv = 1.f / L;
   bf16_t* op = out + ((size_t)(q_begin + j) * Hq + hk * G + (c - j * G)) * HD;
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) {
@@ -555,7 +559,8 @@ __global__ __launch_bounds__(512) void prompt_attention_kernel(
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ block_table, int max_pages, const int* __restrict__ cu_q,
     const int* __restrict__ ctx_len, int Hq, int Hk, int page_size, int page_shift, float scale_log2e,
-    int window, int num_splits, int pair, float* __restrict__ part_o, float* __restrict__ part_ml) {
+    int window, int num_splits, int pair, float* __restrict__ part_o, float* __restrict__ part_ml,
+    const float* __restrict__ sinks) {
   using S = PromptShape<KW>;
   constexpr int TW = S::TW, KB = S::KB, NT = 2, PT = S::PER_THREAD;
   constexpr int VL = PM == 0 ? 2 : 1;                      // loads per 16 bytes of V^T
@@ -970,6 +975,7 @@ __global__ __launch_bounds__(512) void prompt_attention_kernel(
     for (int n = 0; n < NT; ++n) {
       if (!rvalid[n]) continue;
       if (num_splits == 1) {
+        if (sinks) lt[n] += __builtin_amdgcn_exp2f(fmaf(sinks[head[n]], 1.4426950408889634f, -m[n]));
         const float inv = 1.f / lt[n];
         bf16_t* op = out + ((size_t)tok[n] * Hq + head[n]) * HD;
 #pragma unroll
@@ -999,7 +1005,8 @@ template <int KW, int PM>
 static int launch_prompt(dim3 grid, hipStream_t stream, const bf16_t* q, int q_stride, bf16_t* out,
                          const bf16_t* k_pages, const bf16_t* v_pages, const int* block_table, int max_pages,
                          const int* cu_q, const int* ctx_len, int Hq, int Hk, int page_size, int page_shift,
-                         float scale_log2e, int window, int num_splits, int pair, float* part_o, float* part_ml) {
+                         float scale_log2e, int window, int num_splits, int pair, float* part_o, float* part_ml,
+                         const float* sinks) {
   constexpr int lds = PromptShape<KW>::LDS_BYTES;
   static bool sized = false;          // more than 64 KB of LDS has to be asked for, once per kernel
   if (!sized) {
@@ -1010,7 +1017,7 @@ static int launch_prompt(dim3 grid, hipStream_t stream, const bf16_t* q, int q_s
   }
   hipLaunchKernelGGL((prompt_attention_kernel<KW, PM>), grid, dim3(512), lds, stream, q, q_stride, out, k_pages,
                      v_pages, block_table, max_pages, cu_q, ctx_len, Hq, Hk, page_size, page_shift, scale_log2e,
-                     window, num_splits, pair, part_o, part_ml);
+                     window, num_splits, pair, part_o, part_ml, sinks);
   return 0;
 }
 
@@ -1022,7 +1029,8 @@ static int launch_prompt(dim3 grid, hipStream_t stream, const bf16_t* q, int q_s
 template <int S>
 __global__ __launch_bounds__(64) void merge_splits_kernel(const float* __restrict__ part_o,
                                                           const float* __restrict__ part_ml,
-                                                          bf16_t* __restrict__ out, int num_splits) {
+                                                          bf16_t* __restrict__ out, int num_splits,
+                                                          const float* __restrict__ sinks, int Hq) {
   __shared__ float wgt[64];
   const size_t item = blockIdx.x;                 // token * Hq + head
   const int lane = threadIdx.x;
@@ -1042,7 +1050,8 @@ __global__ __launch_bounds__(64) void merge_splits_kernel(const float* __restric
   }
   const float M = wave_max(ms);
   const float w = (ms == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(ms - M);   // an empty split weighs 0
-  const float L = wave_sum(ls * w);
+  float L = wave_sum(ls * w);
+  if (sinks) L += __builtin_amdgcn_exp2f(fmaf(sinks[item % Hq], 1.4426950408889634f, -M));
   wgt[lane] = w;
   __syncthreads();
   const float inv = 1.f / L;
@@ -1066,7 +1075,7 @@ extern "C" int sa_paged_attention_mfma(const void* q, int q_stride, void* out, c
                                        const int* cu_q, const int* ctx_len, int B, int T, int max_q_len,
                                        int Hq, int Hk, int D, int page_size, float scale, int window,
                                        int num_splits, float* part_o, float* part_ml, int in_workgroup,
-                                       hipStream_t stream) {
+                                       const float* sinks, hipStream_t stream) {
   if (T <= 0 || B <= 0) return 0;
   if (D != HD || Hq <= 0 || Hk <= 0 || Hq % Hk || page_size <= 0 || (page_size & 3) || max_pages <= 0 ||
       max_q_len <= 0 || num_splits < 1 || num_splits > 64 || (q_stride & 7))
@@ -1090,7 +1099,7 @@ extern "C" int sa_paged_attention_mfma(const void* q, int q_stride, void* out, c
   hipLaunchKernelGGL((paged_attention_mfma_wg_kernel<PM>), grid, block, 0, stream,                     \
                      (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_pages,                 \
                      (const bf16_t*)v_pages, block_table, max_pages, cu_q, ctx_len, Hq, Hk, page_size, \
-                     page_shift, scale_log2e, window)
+                     page_shift, scale_log2e, window, sinks)
     if (pm == 2) GO(2);
     else if (pm == 1) GO(1);
     else GO(0);
@@ -1106,7 +1115,7 @@ extern "C" int sa_paged_attention_mfma(const void* q, int q_stride, void* out, c
   hipLaunchKernelGGL((paged_attention_mfma_kernel<PM>), grid, block, 0, stream,                        \
                      (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_pages,                 \
                      (const bf16_t*)v_pages, block_table, max_pages, cu_q, ctx_len, Hq, Hk, page_size, \
-                     page_shift, scale_log2e, window, num_splits, part_o, part_ml)
+                     page_shift, scale_log2e, window, num_splits, part_o, part_ml, sinks)
     if (pm == 2) GO(2);
     else if (pm == 1) GO(1);
     else GO(0);
@@ -1128,7 +1137,7 @@ extern "C" int sa_paged_attention_mfma(const void* q, int q_stride, void* out, c
 #define GO(KW, PM)                                                                                       \
   rc = launch_prompt<KW, PM>(grid, stream, (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_pages, \
                              (const bf16_t*)v_pages, block_table, max_pages, cu_q, ctx_len, Hq, Hk, page_size, \
-                             page_shift, scale_log2e, window, num_splits, pair, part_o, part_ml)
+                             page_shift, scale_log2e, window, num_splits, pair, part_o, part_ml, sinks)
     if (kw == 2 && pm == 1) GO(2, 1);
     else if (kw == 2) GO(2, 0);
     else if (pm == 1) GO(4, 1);
@@ -1140,7 +1149,7 @@ extern "C" int sa_paged_attention_mfma(const void* q, int q_stride, void* out, c
   if (num_splits > 1) {
 #define MERGE(S)                                                                                      \
   hipLaunchKernelGGL(merge_splits_kernel<S>, dim3((unsigned)T * Hq), dim3(64), 0, stream, part_o, part_ml, \
-                     (bf16_t*)out, num_splits)
+                     (bf16_t*)out, num_splits, sinks, Hq)
     if (num_splits <= 4) MERGE(4);
     else if (num_splits <= 8) MERGE(8);
     else if (num_splits <= 16) MERGE(16);

@@ -5,7 +5,9 @@
 // prompt portions and single tokens in one launch.  Formulas as in serve/kernels/attn_prefill.py:56-72,205 and attn_decode.py:99-111,236:
 // scores = q.k * scale, key j visible to the query at absolute position p iff j <= p (and
 // p - j < window when a window is set), online softmax (m, l, O), O / l at the end.  Query head
-// h reads KV head h / (Hq / Hk).
+// h reads KV head h / (Hq / Hk).  With `sinks` (fp32 [Hq], or null) the softmax of head h has one more
+// term exp(sinks[h]) in its denominator, which has no key and no value and is not scaled: it joins l
+// when a row is finished (once per row: in the merge where the key range was cut).
 //
 // Batch layout: the T tokens of a step are the concatenation of B segments; segment r covers
 // tokens cu_q[r] .. cu_q[r+1]-1, which are the last q_len positions of a context of ctx_len[r]
@@ -20,7 +22,7 @@ __global__ __launch_bounds__(64) void paged_attention_simple_kernel(
     const TA* __restrict__ q, int q_stride, TA* __restrict__ out, const TC* __restrict__ k_pages,
     const TC* __restrict__ v_pages, const int* __restrict__ block_table, int max_pages,
     const int* __restrict__ cu_q, const int* __restrict__ ctx_len, const int* __restrict__ seg_of_token,
-    int Hq, int Hk, int D, int page_size, float scale, int window, int t0) {
+    int Hq, int Hk, int D, int page_size, float scale, int window, int t0, const float* __restrict__ sinks) {
   __shared__ float qs[SA_MAX_D];
   __shared__ float ps[SA_WAVE];
   __shared__ int vbase_page[SA_WAVE];
@@ -84,6 +86,7 @@ __global__ __launch_bounds__(64) void paged_attention_simple_kernel(
     }
     __syncthreads();
   }
+  if (sinks) l += expf(sinks[h] - m);
   const float inv_l = 1.f / l;
   TA* orow = out + (size_t)t * Hq * D + (size_t)h * D;
 #pragma unroll
@@ -112,7 +115,8 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_f32_kernel(
     const float* __restrict__ q, int q_stride, float* __restrict__ out, const float* __restrict__ k_pages,
     const float* __restrict__ v_pages, const int* __restrict__ block_table, int max_pages,
     const int* __restrict__ cu_q, const int* __restrict__ ctx_len, int Hq, int Hk, int page_size, float scale,
-    int window, int num_splits, float* __restrict__ part_o, float* __restrict__ part_ml) {
+    int window, int num_splits, float* __restrict__ part_o, float* __restrict__ part_ml,
+    const float* __restrict__ sinks) {
   constexpr int D = DV * 16;
   constexpr int LD = D + 4;                       // row length in LDS: keeps 16-byte alignment, spreads banks
   extern __shared__ __attribute__((aligned(16))) float tl_smem[];
@@ -304,7 +308,7 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_f32_kernel(
       }
       continue;
     }
-    const float inv_l = 1.f / l[r];
+    const float inv_l = 1.f / (sinks ? l[r] + expf(sinks[g * G + gi] - m[r]) : l[r]);
     float* orow = out + orow_index * D;
 #pragma unroll
     for (int e = 0; e < DV; ++e) orow[tc + 16 * e] = acc[r][e] * inv_l;
@@ -317,9 +321,10 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_f32_kernel(
 // for one another).
 __global__ __launch_bounds__(64) void paged_attention_merge_f32_kernel(const float* __restrict__ part_o,
                                                                        const float* __restrict__ part_ml,
-                                                                       float* __restrict__ out, int D, int num_splits) {
+                                                                       float* __restrict__ out, int D, int num_splits,
+                                                                       const float* __restrict__ sinks, int Hq) {
   __shared__ float wgt[64];
-  const size_t row = blockIdx.x;
+  const size_t row = blockIdx.x;                  // (token, head)
   const int lane = threadIdx.x;
   float ms = -INFINITY, ls = 0.f;
   if (lane < num_splits) {
@@ -328,7 +333,9 @@ __global__ __launch_bounds__(64) void paged_attention_merge_f32_kernel(const flo
   }
   const float mx = wave_max(ms);
   const float w = ms == -INFINITY ? 0.f : expf(ms - mx);
-  const float inv = 1.f / wave_sum(w * ls);
+  float total = wave_sum(w * ls);
+  if (sinks) total += expf(sinks[row % Hq] - mx);
+  const float inv = 1.f / total;
   wgt[lane] = w;
   __syncthreads();
   const float* po = part_o + row * num_splits * D;
@@ -344,7 +351,7 @@ template <int DV>
 static int launch_tiled(const void* q, int q_stride, void* out, const void* k_pages, const void* v_pages,
                         const int* block_table, int max_pages, const int* cu_q, const int* ctx_len, int B,
                         int max_q_len, int Hq, int Hk, int page_size, float scale, int window, int num_splits,
-                        float* part_o, float* part_ml, hipStream_t stream) {
+                        float* part_o, float* part_ml, const float* sinks, hipStream_t stream) {
   constexpr int D = DV * 16;
   const size_t lds = (size_t)(3 * 64 * (D + 4) + 64 * 68) * sizeof(float);
   const long long items = ((long long)max_q_len * (Hq / Hk) + TL_ROWS - 1) / TL_ROWS;
@@ -355,7 +362,7 @@ static int launch_tiled(const void* q, int q_stride, void* out, const void* k_pa
   dim3 grid((unsigned)(items * Hk), B * num_splits), block(256);
   hipLaunchKernelGGL((paged_attention_tiled_f32_kernel<DV>), grid, block, lds, stream, (const float*)q, q_stride,
                      (float*)out, (const float*)k_pages, (const float*)v_pages, block_table, max_pages, cu_q,
-                     ctx_len, Hq, Hk, page_size, scale, window, num_splits, part_o, part_ml);
+                     ctx_len, Hq, Hk, page_size, scale, window, num_splits, part_o, part_ml, sinks);
   SA_LAUNCH_CHECK();
   return 0;
 }
@@ -379,7 +386,8 @@ __global__ __launch_bounds__(64) void paged_attention_decode_f32_kernel(
     const float* __restrict__ q, int q_stride, float* __restrict__ out, const float* __restrict__ k_pages,
     const float* __restrict__ v_pages, const int* __restrict__ block_table, int max_pages,
     const int* __restrict__ cu_q, const int* __restrict__ ctx_len, int Hq, int Hk, int page_size, float scale,
-    int window, int num_splits, float* __restrict__ part_o, float* __restrict__ part_ml) {
+    int window, int num_splits, float* __restrict__ part_o, float* __restrict__ part_ml,
+    const float* __restrict__ sinks) {
   constexpr int D = DV * 16;
   constexpr int NA = (D + 63) / 64;               // dims per lane in the product with V
   __shared__ __attribute__((aligned(16))) float ps[GR][64];
@@ -511,6 +519,7 @@ __global__ __launch_bounds__(64) void paged_attention_decode_f32_kernel(
   for (int r = 0; r < GR; ++r) {
     if (h0 + r >= G) continue;
     const size_t row = (size_t)t * Hq + g * G + h0 + r;           // (token, head)
+    if (sinks && num_splits == 1) l[r] += expf(sinks[g * G + h0 + r] - m[r]);
 #pragma unroll
     for (int a = 0; a < NA; ++a) {
       const int d = lane + 64 * a;
@@ -529,7 +538,7 @@ template <int DV>
 static int launch_decode_f32(const void* q, int q_stride, void* out, const void* k_pages, const void* v_pages,
                              const int* block_table, int max_pages, const int* cu_q, const int* ctx_len, int B,
                              int Hq, int Hk, int page_size, float scale, int window, int num_splits, float* part_o,
-                             float* part_ml, hipStream_t stream) {
+                             float* part_ml, const float* sinks, hipStream_t stream) {
   const int G = Hq / Hk;
   const int gr = G >= 3 ? 4 : G;                  // heads per wave: 1, 2 or 4
   const long long gx = (long long)Hk * ((G + gr - 1) / gr);
@@ -538,7 +547,7 @@ static int launch_decode_f32(const void* q, int q_stride, void* out, const void*
 #define GO(GR)                                                                                                    \
   hipLaunchKernelGGL((paged_attention_decode_f32_kernel<DV, GR>), grid, block, 0, stream, (const float*)q,        \
                      q_stride, (float*)out, (const float*)k_pages, (const float*)v_pages, block_table, max_pages, \
-                     cu_q, ctx_len, Hq, Hk, page_size, scale, window, num_splits, part_o, part_ml)
+                     cu_q, ctx_len, Hq, Hk, page_size, scale, window, num_splits, part_o, part_ml, sinks)
   if (gr == 1) GO(1);
   else if (gr == 2) GO(2);
   else GO(4);
@@ -558,7 +567,7 @@ extern "C" int sa_paged_attention_decode_f32(const void* q, int q_stride, void* 
                                              const void* v_pages, const int* block_table, int max_pages,
                                              const int* cu_q, const int* ctx_len, int B, int first_token, int Hq,
                                              int Hk, int D, int page_size, float scale, int window, int num_splits,
-                                             float* part_o, float* part_ml, hipStream_t stream) {
+                                             float* part_o, float* part_ml, const float* sinks, hipStream_t stream) {
   if (B <= 0) return 0;
   if (Hq <= 0 || Hk <= 0 || Hq % Hk || D <= 0 || D > 128 || (D & 15) || page_size <= 0 || (page_size & 3) ||
       max_pages <= 0 || (q_stride & 3) || num_splits < 1 || num_splits > 64 || first_token < 0)
@@ -568,7 +577,7 @@ extern "C" int sa_paged_attention_decode_f32(const void* q, int q_stride, void* 
 #define GO(DV)                                                                                                   \
   case DV:                                                                                                       \
     rc = launch_decode_f32<DV>(q, q_stride, out, k_pages, v_pages, block_table, max_pages, cu_q, ctx_len, B, Hq, \
-                               Hk, page_size, scale, window, num_splits, part_o, part_ml, stream);               \
+                               Hk, page_size, scale, window, num_splits, part_o, part_ml, sinks, stream);        \
     break
   switch (D / 16) {
     GO(1);
@@ -585,7 +594,7 @@ extern "C" int sa_paged_attention_decode_f32(const void* q, int q_stride, void* 
   const size_t row0 = (size_t)first_token * Hq;
   hipLaunchKernelGGL(paged_attention_merge_f32_kernel, dim3((unsigned)B * Hq), dim3(64), 0, stream,
                      part_o + row0 * num_splits * D, part_ml + row0 * num_splits * 2, (float*)out + row0 * D, D,
-                     num_splits);
+                     num_splits, sinks, Hq);
   SA_LAUNCH_CHECK();
   return 0;
 }
@@ -599,7 +608,8 @@ extern "C" int sa_paged_attention_tiled_f32(const void* q, int q_stride, void* o
                                             const void* v_pages, const int* block_table, int max_pages,
                                             const int* cu_q, const int* ctx_len, int B, int T, int max_q_len,
                                             int Hq, int Hk, int D, int page_size, float scale, int window,
-                                            int num_splits, float* part_o, float* part_ml, hipStream_t stream) {
+                                            int num_splits, float* part_o, float* part_ml, const float* sinks,
+                                            hipStream_t stream) {
   if (B <= 0 || max_q_len <= 0 || T <= 0) return 0;
   if (Hq <= 0 || Hk <= 0 || Hq % Hk || D <= 0 || D > 128 || (D & 15) || page_size <= 0 || (page_size & 3) ||
       max_pages <= 0 || (q_stride & 3) || num_splits < 1 || num_splits > 64)
@@ -609,7 +619,8 @@ extern "C" int sa_paged_attention_tiled_f32(const void* q, int q_stride, void* o
 #define GO(DV)                                                                                                  \
   case DV:                                                                                                      \
     rc = launch_tiled<DV>(q, q_stride, out, k_pages, v_pages, block_table, max_pages, cu_q, ctx_len, B,         \
-                          max_q_len, Hq, Hk, page_size, scale, window, num_splits, part_o, part_ml, stream);    \
+                          max_q_len, Hq, Hk, page_size, scale, window, num_splits, part_o, part_ml, sinks,     \
+                          stream);                                                                              \
     break
   switch (D / 16) {
     GO(1);
@@ -624,7 +635,7 @@ extern "C" int sa_paged_attention_tiled_f32(const void* q, int q_stride, void* o
 #undef GO
   if (rc != 0 || num_splits == 1) return rc;
   hipLaunchKernelGGL(paged_attention_merge_f32_kernel, dim3((unsigned)T * Hq), dim3(64), 0, stream, part_o, part_ml,
-                     (float*)out, D, num_splits);
+                     (float*)out, D, num_splits, sinks, Hq);
   SA_LAUNCH_CHECK();
   return 0;
 }
@@ -634,7 +645,7 @@ extern "C" int sa_paged_attention_simple(const void* q, int q_stride, void* out,
                                          const int* block_table, int max_pages, const int* cu_q,
                                          const int* ctx_len, const int* seg_of_token, int T, int Hq,
                                          int Hk, int D, int page_size, float scale, int window,
-                                         hipStream_t stream) {
+                                         const float* sinks, hipStream_t stream) {
   if (T <= 0) return 0;
   if (Hq <= 0 || Hk <= 0 || Hq % Hk || D <= 0 || D > SA_MAX_D || page_size <= 0 || max_pages <= 0)
     return SA_ERR_ARG;
@@ -648,7 +659,7 @@ extern "C" int sa_paged_attention_simple(const void* q, int q_stride, void* out,
   hipLaunchKernelGGL((paged_attention_simple_kernel<TA, TC>), grid, block, 0, stream,                \
                      (const TA*)q, q_stride, (TA*)out, (const TC*)k_pages, (const TC*)v_pages,       \
                      block_table, max_pages, cu_q, ctx_len, seg_of_token, Hq, Hk, D, page_size,     \
-                     scale, window, t0)
+                     scale, window, t0, sinks)
     if (act_dtype == SA_F32 && cache_dtype == SA_F32) GO(float, float);
     else if (act_dtype == SA_BF16 && cache_dtype == SA_BF16) GO(bf16_t, bf16_t);
     else return SA_ERR_UNSUPPORTED;

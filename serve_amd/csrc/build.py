@@ -48,6 +48,7 @@ SOURCES: Dict[str, str] = {
     "delta_rule": "delta_rule.hip",
     "latent": "latent.hip",
     "moe": "moe.hip",
+    "qk_norm": "qk_norm.hip",
 }
 # what a library is linked with beside the HIP runtime
 LINK: Dict[str, List[str]] = {"blaslt.hip": ["-lhipblaslt"]}

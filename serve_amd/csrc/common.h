@@ -69,6 +69,23 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
   return t;
 }
 
+// Gated feed-forwards multiply an activated "gate" branch with a second, linear branch:
+//   silu           g sigmoid(g) * u
+//   gelu_tanh      0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))) * u
+//   clamped_swish  g' sigmoid(1.702 g') * (u' + 1), g' = min(g, limit), u' = clamp(u, -limit, limit)
+enum { SA_GATE_SILU = 0, SA_GATE_GELU_TANH = 1, SA_GATE_CLAMPED_SWISH = 2, SA_GATE_KINDS = 3 };
+
+__device__ __forceinline__ float gate_mul(float g, float u, int kind, float limit) {
+  if (kind == SA_GATE_GELU_TANH)
+    return (0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)))) * u;
+  if (kind == SA_GATE_CLAMPED_SWISH) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return (g / (1.f + expf(-1.702f * g))) * (u + 1.f);
+  }
+  return (g / (1.f + expf(-g))) * u;
+}
+
 // sin and cos of an angle of up to 4e6 rad (a position times a frequency of at most 1), to about
 // 1e-6: the library's sincosf spends over a thousand cycles on arguments this large.  The multiple
 // of 2 pi is taken off in three steps whose constants have few enough bits for the first two

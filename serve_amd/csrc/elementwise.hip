@@ -11,19 +11,19 @@
 template <typename TW>
 __global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict__ tokens,
                              const int* __restrict__ src_row, const int* __restrict__ prev,
-                             float* __restrict__ x, int d, int V) {
+                             float* __restrict__ x, int d, int V, float scale) {
   const int t = blockIdx.x;
   int tok = tokens[t];
   if (src_row && src_row[t] >= 0) tok = prev[src_row[t]];
   tok = min(max(tok, 0), V - 1);
   const size_t row = (size_t)tok * (size_t)d;
-  for (int i = threadIdx.x; i < d; i += blockDim.x) x[(size_t)t * d + i] = to_float(table[row + i]);
+  for (int i = threadIdx.x; i < d; i += blockDim.x) x[(size_t)t * d + i] = to_float(table[row + i]) * scale;
 }
 
 // bf16 rows of whole groups of eight from aligned addresses: 16 bytes a lane in, two times 16 out
 __global__ __launch_bounds__(256) void embed_bf16x8_kernel(const bf16_t* __restrict__ table, const int* __restrict__ tokens,
                                                             const int* __restrict__ src_row, const int* __restrict__ prev,
-                                                            float* __restrict__ x, int d, int V) {
+                                                            float* __restrict__ x, int d, int V, float scale) {
   const int t = blockIdx.x;
   int tok = tokens[t];
   if (src_row && src_row[t] >= 0) tok = prev[src_row[t]];
@@ -36,8 +36,8 @@ __global__ __launch_bounds__(256) void embed_bf16x8_kernel(const bf16_t* __restr
     float f[8];
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-      f[2 * k] = bf16_bits_to_float(w[k] & 0xffffu);
-      f[2 * k + 1] = bf16_bits_to_float(w[k] >> 16);
+      f[2 * k] = bf16_bits_to_float(w[k] & 0xffffu) * scale;
+      f[2 * k + 1] = bf16_bits_to_float(w[k] >> 16) * scale;
     }
     *reinterpret_cast<float4*>(out + i) = make_float4(f[0], f[1], f[2], f[3]);
     *reinterpret_cast<float4*>(out + i + 4) = make_float4(f[4], f[5], f[6], f[7]);
@@ -45,22 +45,22 @@ __global__ __launch_bounds__(256) void embed_bf16x8_kernel(const bf16_t* __restr
 }
 
 extern "C" int sa_embed(const void* table, int table_dtype, const int* tokens, const int* src_row,
-                        const int* prev, float* x, int T, int d, int V, hipStream_t stream) {
+                        const int* prev, float* x, int T, int d, int V, float scale, hipStream_t stream) {
   if (T <= 0) return 0;
   if (d <= 0 || V <= 0 || (src_row && !prev)) return SA_ERR_ARG;
   dim3 grid(T), block(256);
   if (table_dtype == SA_BF16 && (d & 7) == 0 && ((uintptr_t)table & 15) == 0 && ((uintptr_t)x & 15) == 0) {
     hipLaunchKernelGGL(embed_bf16x8_kernel, grid, block, 0, stream, (const bf16_t*)table, tokens, src_row, prev, x,
-                       d, V);
+                       d, V, scale);
     SA_LAUNCH_CHECK();
     return 0;
   }
   if (table_dtype == SA_F32)
     hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, (const float*)table, tokens, src_row, prev,
-                       x, d, V);
+                       x, d, V, scale);
   else if (table_dtype == SA_BF16)
     hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)table, tokens, src_row, prev,
-                       x, d, V);
+                       x, d, V, scale);
   else
     return SA_ERR_UNSUPPORTED;
   SA_LAUNCH_CHECK();
@@ -389,22 +389,22 @@ extern "C" int sa_rope_kv_write(void* qkv, int act_dtype, const int* positions, 
 }
 
 // ---------------------------------------------------------------------------------------------
-// SwiGLU gate (serve/model.py:85): a[t, i] = silu(gu[t, i]) * gu[t, I + i]
+// SwiGLU gate (serve/model.py:85): a[t, i] = silu(gu[t, i]) * gu[t, I + i]; or another gate (gate_mul)
 // ---------------------------------------------------------------------------------------------
 template <typename TA>
-__global__ void silu_mul_kernel(const TA* __restrict__ gu, TA* __restrict__ a, int T, int I) {
+__global__ void silu_mul_kernel(const TA* __restrict__ gu, TA* __restrict__ a, int T, int I, int kind, float limit) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= I) return;
   for (int t = blockIdx.y; t < T; t += gridDim.y) {
     const float g = to_float(gu[(size_t)t * 2 * I + i]);
     const float u = to_float(gu[(size_t)t * 2 * I + I + i]);
-    a[(size_t)t * I + i] = from_float<TA>((g / (1.f + expf(-g))) * u);
+    a[(size_t)t * I + i] = from_float<TA>(gate_mul(g, u, kind, limit));
   }
 }
 
 // the same, eight bf16 values per thread in 16-byte vectors (I % 8 == 0)
 __global__ __launch_bounds__(256) void silu_mul_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ a,
-                                                               int T, int I) {
+                                                               int T, int I, int kind, float limit) {
   const int i = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
   if (i >= I) return;
   for (int t = blockIdx.y; t < T; t += gridDim.y) {
@@ -417,28 +417,29 @@ __global__ __launch_bounds__(256) void silu_mul_bf16x8_kernel(const bf16_t* __re
     for (int k = 0; k < 4; ++k) {
       const float g0 = bf16_bits_to_float(gw[k] & 0xffffu), g1 = bf16_bits_to_float(gw[k] >> 16);
       const float u0 = bf16_bits_to_float(uw[k] & 0xffffu), u1 = bf16_bits_to_float(uw[k] >> 16);
-      const float o0 = (g0 / (1.f + expf(-g0))) * u0;
-      const float o1 = (g1 / (1.f + expf(-g1))) * u1;
+      const float o0 = gate_mul(g0, u0, kind, limit);
+      const float o1 = gate_mul(g1, u1, kind, limit);
       ow[k] = (uint32_t)float_to_bf16_bits(o0) | ((uint32_t)float_to_bf16_bits(o1) << 16);
     }
     *reinterpret_cast<uint4*>(a + (size_t)t * I + i) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
   }
 }
 
-extern "C" int sa_silu_mul(const void* gu, void* a, int act_dtype, int T, int I, hipStream_t stream) {
+extern "C" int sa_gate_mul(const void* gu, void* a, int act_dtype, int T, int I, int kind, float limit,
+                           hipStream_t stream) {
   if (T <= 0) return 0;
-  if (I <= 0) return SA_ERR_ARG;
+  if (I <= 0 || kind < 0 || kind >= SA_GATE_KINDS) return SA_ERR_ARG;
   if (act_dtype == SA_BF16 && (I & 7) == 0) {
     dim3 grid((I / 8 + 255) / 256, T < 32768 ? T : 32768), block(256);
-    hipLaunchKernelGGL(silu_mul_bf16x8_kernel, grid, block, 0, stream, (const bf16_t*)gu, (bf16_t*)a, T, I);
+    hipLaunchKernelGGL(silu_mul_bf16x8_kernel, grid, block, 0, stream, (const bf16_t*)gu, (bf16_t*)a, T, I, kind, limit);
     SA_LAUNCH_CHECK();
     return 0;
   }
   dim3 grid((I + 255) / 256, T < 32768 ? T : 32768), block(256);
   if (act_dtype == SA_F32)
-    hipLaunchKernelGGL(silu_mul_kernel<float>, grid, block, 0, stream, (const float*)gu, (float*)a, T, I);
+    hipLaunchKernelGGL(silu_mul_kernel<float>, grid, block, 0, stream, (const float*)gu, (float*)a, T, I, kind, limit);
   else if (act_dtype == SA_BF16)
-    hipLaunchKernelGGL(silu_mul_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)gu, (bf16_t*)a, T, I);
+    hipLaunchKernelGGL(silu_mul_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)gu, (bf16_t*)a, T, I, kind, limit);
   else
     return SA_ERR_UNSUPPORTED;
   SA_LAUNCH_CHECK();

@@ -1,5 +1,7 @@
 // Routed experts: every token takes the `top` experts with the largest router logits, weighted by the
-// softmax over those logits alone; an expert is down(silu(gate x) * up x).
+// softmax over those logits alone (or: by their shares of the softmax over all experts, divided by the sum
+// of the chosen shares + 1e-20; either way times a constant); an expert is down(gate(gate x, up x)) with
+// one of the gates of common.h (silu(g) u and others).
 //
 // Nothing is read back to the host: the tokens are grouped by expert on the device, and the
 // products run over a list of (expert, rows) tiles that is built there, from a grid sized for
@@ -23,19 +25,22 @@
 // ---------------------------------------------------------------------------------------------
 // route: a wave per token.  Ties go to the lower index.
 // ---------------------------------------------------------------------------------------------
+// over_all: the weights are shares of the softmax over all E logits, renormalised over the chosen ones
+// (p_k / S) / (sum_chosen p / S + 1e-20) with S the sum over all; else p_k / sum_chosen p.  Both times wscale.
 __device__ __forceinline__ void route_token(const float* __restrict__ z, int* __restrict__ ids, float* __restrict__ wts,
-                                            int E, int top, int lane);
+                                            int E, int top, int lane, int over_all, float wscale);
 
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int ldz, int* __restrict__ ids,
-                                                        float* __restrict__ wts, int T, int E, int top) {
+                                                        float* __restrict__ wts, int T, int E, int top, int over_all,
+                                                        float wscale) {
   const int t = blockIdx.x * (blockDim.x / SA_WAVE) + threadIdx.x / SA_WAVE;
   if (t >= T) return;
   route_token(logits + (size_t)t * ldz, ids + (size_t)t * top, wts + (size_t)t * top, E, top,
-              threadIdx.x & (SA_WAVE - 1));
+              threadIdx.x & (SA_WAVE - 1), over_all, wscale);
 }
 
 __device__ __forceinline__ void route_token(const float* __restrict__ z, int* __restrict__ ids, float* __restrict__ wts,
-                                            int E, int top, int lane) {
+                                            int E, int top, int lane, int over_all, float wscale) {
   float prev_v = INFINITY;
   int prev_i = -1;
   float first = 0.f, sum = 0.f;
@@ -64,8 +69,17 @@ __device__ __forceinline__ void route_token(const float* __restrict__ z, int* __
     prev_v = bv;
     prev_i = bi;
   }
-  if (lane == 0)
-    for (int k = 0; k < top; ++k) wts[k] /= sum;
+  float all = 1.f;
+  if (over_all) {
+    // the softmax's denominator over every expert, with the largest logit taken off
+    float part = 0.f;
+    for (int e = lane; e < E; e += SA_WAVE) part += expf(z[e] - first);
+    all = wave_sum(part);
+  }
+  if (lane == 0) {
+    const float denom = over_all ? sum / all + 1e-20f : sum;
+    for (int k = 0; k < top; ++k) wts[k] = ((over_all ? wts[k] / all : wts[k]) / denom) * wscale;
+  }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -78,14 +92,14 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int* ids, int n, 
                                                          int* __restrict__ perm, int* __restrict__ tile_expert,
                                                          int* __restrict__ tile_row0, int* __restrict__ num_tiles,
                                                          const float* __restrict__ logits, int ldz, int* ids_out,
-                                                         float* __restrict__ wts, int top) {
+                                                         float* __restrict__ wts, int top, int over_all, float wscale) {
   for (int e = threadIdx.x; e < E; e += blockDim.x) cursor[e] = 0;
   if (logits) {
     // a step of few tokens: the routing is done here, a wave a token in turn, and saves a kernel
     const int waves = blockDim.x / SA_WAVE, T = n / top;
     for (int t = threadIdx.x / SA_WAVE; t < T; t += waves)
       route_token(logits + (size_t)t * ldz, ids_out + (size_t)t * top, wts + (size_t)t * top, E, top,
-                  threadIdx.x & (SA_WAVE - 1));
+                  threadIdx.x & (SA_WAVE - 1), over_all, wscale);
   }
   __syncthreads();
   for (int i = threadIdx.x; i < n; i += blockDim.x) atomicAdd(&cursor[ids[i]], 1);
@@ -161,7 +175,8 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(const TA* __restrict__
                                                           const TA* __restrict__ Wu, const int* __restrict__ offsets,
                                                           const int* __restrict__ perm, const int* __restrict__ tile_expert,
                                                           const int* __restrict__ tile_row0, const int* __restrict__ num_tiles,
-                                                          TA* __restrict__ act, int top, int d, int F) {
+                                                          TA* __restrict__ act, int top, int d, int F, int gate_kind,
+                                                          float gate_limit) {
   __shared__ float sa[MOE_TK][MOE_TM + 1];
   __shared__ float sw0[MOE_TK][MOE_TN + 1];
   __shared__ float sw1[MOE_TK][MOE_TN + 1];
@@ -184,8 +199,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(const TA* __restrict__
     for (int c = 0; c < 4; ++c) {
       const int n = n0 + tx + 16 * c;
       if (n < F) {
-        const float gv = g[rr][c];
-        act[(size_t)(row0 + r) * F + n] = from_float<TA>((gv / (1.f + expf(-gv))) * u[rr][c]);
+        act[(size_t)(row0 + r) * F + n] = from_float<TA>(gate_mul(g[rr][c], u[rr][c], gate_kind, gate_limit));
       }
     }
   }
@@ -233,7 +247,7 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const TA* __restrict__ ac
 //            and walk all of K (prompt portions: an expert's matrix is read once per 16 MT rows).
 //   KS == 4: tiles of up to 16 rows (MT 1); the four waves cut K between them and add through LDS in a
 //            fixed order (decode steps: few rows per expert, the chip is filled by cutting K and N).
-// GATE_UP: rows come from h by perm[row] / top, two matrices, act = silu(gate) * up in bf16.
+// GATE_UP: rows come from h by perm[row] / top, two matrices, act = gate(gate, up) in bf16.
 // else:    rows are act's own, one matrix, fp32 sums go to yk[perm[row]].
 // ---------------------------------------------------------------------------------------------
 typedef __bf16 moe_bf16x8_t __attribute__((ext_vector_type(8)));
@@ -250,7 +264,7 @@ __global__ __launch_bounds__(256) void moe_mfma_kernel(const bf16_t* __restrict_
                                                        const int* __restrict__ perm, const int* __restrict__ tile_expert,
                                                        const int* __restrict__ tile_row0, const int* __restrict__ num_tiles,
                                                        bf16_t* __restrict__ act, float* __restrict__ yk, int top, int N,
-                                                       int K) {
+                                                       int K, int gate_kind, float gate_limit) {
   // WR: groups of 16 weight rows a wave owns (per matrix); KU: steps of 32 along K whose loads are in flight together
   constexpr int NM = GATE_UP ? 2 : 1;
   constexpr int RT = NM * WR;
@@ -345,10 +359,8 @@ __global__ __launch_bounds__(256) void moe_mfma_kernel(const bf16_t* __restrict_
         bf16_t* dst = act + (size_t)(row0 + m) * N + n;
 #pragma unroll
         for (int r = 0; r < 4; ++r)
-          if (n + r < N) {
-            const float gv = acc[wr][mt][r];
-            dst[r] = from_float<bf16_t>((gv / (1.f + expf(-gv))) * acc[RT - WR + wr][mt][r]);
-          }
+          if (n + r < N)
+            dst[r] = from_float<bf16_t>(gate_mul(acc[wr][mt][r], acc[RT - WR + wr][mt][r], gate_kind, gate_limit));
       } else {
         float* dst = yk + (size_t)perm[row0 + m] * N + n;
 #pragma unroll
@@ -406,11 +418,11 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
 extern "C" int sa_moe_max_tiles(int rows, int E) { return (rows + 15) / 16 + E; }
 
 extern "C" int sa_moe_route(const float* logits, int ldz, int* ids, float* wts, int T, int E, int top,
-                            hipStream_t stream) {
+                            int over_all, float wscale, hipStream_t stream) {
   if (T <= 0) return 0;
   if (E <= 0 || top <= 0 || top > E || ldz < E) return SA_ERR_ARG;
   dim3 grid((T + 3) / 4), block(256);
-  hipLaunchKernelGGL(moe_route_kernel, grid, block, 0, stream, logits, ldz, ids, wts, T, E, top);
+  hipLaunchKernelGGL(moe_route_kernel, grid, block, 0, stream, logits, ldz, ids, wts, T, E, top, over_all, wscale);
   SA_LAUNCH_CHECK();
   return 0;
 }
@@ -427,10 +439,12 @@ extern "C" int sa_moe_route_inside_limit() { return MOE_ROUTE_INSIDE; }
 
 extern "C" int sa_moe_experts(const void* h, int act_dtype, int* ids, const void* Wg, const void* Wu,
                               const void* Wd, int* ints, void* act, float* yk, int T, int top, int E, int d, int F,
-                              const float* logits, int ldz, float* wts, hipStream_t stream) {
+                              const float* logits, int ldz, float* wts, int over_all, float wscale, int gate_kind,
+                              float gate_limit, hipStream_t stream) {
   if (T <= 0) return 0;
   const long long n = (long long)T * top;
   if (E <= 0 || top <= 0 || d <= 0 || F <= 0 || n > 0x3fffffffLL) return SA_ERR_ARG;
+  if (gate_kind < 0 || gate_kind >= SA_GATE_KINDS) return SA_ERR_ARG;
   const int max_tiles = sa_moe_max_tiles((int)n, E);
   int* offsets = ints;
   int* cursor = offsets + E + 1;
@@ -444,7 +458,7 @@ extern "C" int sa_moe_experts(const void* h, int act_dtype, int* ids, const void
   const int tiles = (int)((n + tile_rows - 1) / tile_rows) + E;
   if (logits && (T > MOE_ROUTE_INSIDE || !wts || ldz < E || top > E)) return SA_ERR_ARG;
   hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), 0, stream, ids, (int)n, E, tile_rows, offsets, cursor, perm,
-                     tile_expert, tile_row0, num_tiles, logits, ldz, ids, wts, top);
+                     tile_expert, tile_row0, num_tiles, logits, ldz, ids, wts, top, over_all, wscale);
   SA_LAUNCH_CHECK();
   dim3 block(256);
   if (mfma) {
@@ -458,10 +472,10 @@ extern "C" int sa_moe_experts(const void* h, int act_dtype, int* ids, const void
   do {                                                                                                                 \
     hipLaunchKernelGGL((moe_mfma_kernel<MT, KS, true, WR, KU>), g1, block, 0, stream, (const bf16_t*)h, (const bf16_t*)Wg,     \
                        (const bf16_t*)Wu, offsets, perm, tile_expert, tile_row0, num_tiles, (bf16_t*)act, nullptr,     \
-                       top, F, d);                                                                                     \
+                       top, F, d, gate_kind, gate_limit);                                                              \
     SA_LAUNCH_CHECK();                                                                                                 \
     hipLaunchKernelGGL((moe_mfma_kernel<MT, KS, false, WR, KU>), g2, block, 0, stream, (const bf16_t*)act, (const bf16_t*)Wd,  \
-                       nullptr, offsets, perm, tile_expert, tile_row0, num_tiles, nullptr, yk, top, d, F);             \
+                       nullptr, offsets, perm, tile_expert, tile_row0, num_tiles, nullptr, yk, top, d, F, 0, 0.f);     \
   } while (0)
     if (small) GO(1, 4, 1, 2);
     else GO(4, 1, 4, 2);
@@ -473,13 +487,15 @@ extern "C" int sa_moe_experts(const void* h, int act_dtype, int* ids, const void
   if (g1.y > 65535 || g2.y > 65535) return SA_ERR_ARG;
   if (act_dtype == SA_F32) {
     hipLaunchKernelGGL(moe_gate_up_kernel<float>, g1, block, 0, stream, (const float*)h, (const float*)Wg,
-                       (const float*)Wu, offsets, perm, tile_expert, tile_row0, num_tiles, (float*)act, top, d, F);
+                       (const float*)Wu, offsets, perm, tile_expert, tile_row0, num_tiles, (float*)act, top, d, F,
+                       gate_kind, gate_limit);
     SA_LAUNCH_CHECK();
     hipLaunchKernelGGL(moe_down_kernel<float>, g2, block, 0, stream, (const float*)act, (const float*)Wd, offsets, perm,
                        tile_expert, tile_row0, num_tiles, yk, d, F);
   } else if (act_dtype == SA_BF16) {
     hipLaunchKernelGGL(moe_gate_up_kernel<bf16_t>, g1, block, 0, stream, (const bf16_t*)h, (const bf16_t*)Wg,
-                       (const bf16_t*)Wu, offsets, perm, tile_expert, tile_row0, num_tiles, (bf16_t*)act, top, d, F);
+                       (const bf16_t*)Wu, offsets, perm, tile_expert, tile_row0, num_tiles, (bf16_t*)act, top, d, F,
+                       gate_kind, gate_limit);
     SA_LAUNCH_CHECK();
     hipLaunchKernelGGL(moe_down_kernel<bf16_t>, g2, block, 0, stream, (const bf16_t*)act, (const bf16_t*)Wd, offsets,
                        perm, tile_expert, tile_row0, num_tiles, yk, d, F);

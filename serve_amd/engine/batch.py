@@ -78,6 +78,10 @@ class StepContext:
     # the residual stream in the activation dtype, where the layer that ran last has made that copy and
     # the stream has not changed since (layers whose sublayers read the stream itself pass it on)
     stream_copy: Optional[torch.Tensor] = None
+    # what a layer leaves for later layers of the same step, by name (the first layer's values that later
+    # layers blend with theirs, a normed stream made ahead for the layer that reads it); emptied by the model
+    # at the start of a step
+    shared: dict = field(default_factory=dict)
 
 
 def _align(n: int) -> int:

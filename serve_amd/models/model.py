@@ -166,6 +166,7 @@ class Model:
         """Run the tokens of one step; return fp32 logits [R, V] at ctx.logit_rows."""
         x = self.embedding.forward(ctx)
         ctx.stream_copy = None          # (what a layer may leave for the next: the stream in the activation dtype)
+        ctx.shared = {}                 # (and what layers leave for later layers of the step, by name)
         pending = None
         for e in self.spec.run_order:
             pending = self.layers[e.layer].forward(x, pending, ctx, caches[e.cache], e.writes_cache)

@@ -92,8 +92,9 @@ def _i32(t: torch.Tensor, n: int, name: str) -> None:
 # ---------------------------------------------------------------------------------------------
 
 def embed(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor,
-          src_row: Optional[torch.Tensor] = None, prev: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out[t] = table[tokens[t]] as fp32.  Where src_row[t] >= 0 the id is prev[src_row[t]] instead:
+          src_row: Optional[torch.Tensor] = None, prev: Optional[torch.Tensor] = None,
+          scale: float = 1.0) -> torch.Tensor:
+    """out[t] = table[tokens[t]] * scale as fp32 (the product is taken in fp32).  Where src_row[t] >= 0 the id is prev[src_row[t]] instead:
     a token sampled on the device by an earlier step.  Host-given ids have been checked against
     the table by the batch builder; the kernel clamps as a last resort."""
     _dev(table, tokens, out, src_row, prev)
@@ -107,7 +108,7 @@ def embed(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor,
         _check(prev is not None and prev.dtype == torch.int32, "prev must be int32")
     lib = load_library("elementwise")
     _ret(lib.sa_embed(_ptr(table), c_int(_code(table)), _ptr(tokens), _ptr(src_row), _ptr(prev), _ptr(out),
-                      c_int(T), c_int(d), c_int(V), _stream()), "embed")
+                      c_int(T), c_int(d), c_int(V), c_float(scale), _stream()), "embed")
     return out
 
 
@@ -233,15 +234,25 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Te
 SIMPLE_ATTENTION_MAX_HEAD_DIM = 640     # (SA_MAX_D of csrc/attention_simple.hip)
 
 
+def _check_sinks(sinks: Optional[torch.Tensor], num_heads: int) -> None:
+    """`sinks`: per query head one more term exp(sinks[h]) in the softmax's denominator, with no key and
+    no value (fp32 [Hq] on the device); None: a plain softmax."""
+    if sinks is not None:
+        _check(sinks.is_cuda and sinks.is_contiguous() and sinks.dtype == torch.float32
+               and sinks.numel() == num_heads, f"sinks must be contiguous fp32 [{num_heads}] on the GPU")
+
+
 def paged_attention_simple(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pages: torch.Tensor,
                            v_pages: torch.Tensor, block_table: torch.Tensor, cu_q: torch.Tensor,
                            ctx_len: torch.Tensor, seg_of_token: torch.Tensor, num_tokens: int,
-                           num_heads: int, scale: float, window: Optional[int]) -> torch.Tensor:
+                           num_heads: int, scale: float, window: Optional[int],
+                           sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of every token of the step over its request's cached keys (fp32 arithmetic), a wave
     per (token, head): the general form, for sizes that the other kernels do not take.
 
     q is the start of the q block of the fused qkv rows (row stride `q_row_stride` elements)."""
     _dev(q, out, k_pages, v_pages, block_table, cu_q, ctx_len, seg_of_token)
+    _check_sinks(sinks, num_heads)
     P, Hk, page_size, D = k_pages.shape
     _check(v_pages.shape == (P, Hk, D, page_size), "v_pages must be [P, Hk, D, page_size]")
     _check(num_heads % Hk == 0, "query heads must be a multiple of KV heads")
@@ -260,7 +271,7 @@ def paged_attention_simple(q: torch.Tensor, q_row_stride: int, out: torch.Tensor
         _ptr(q), c_int(q_row_stride), _ptr(out), c_int(_code(q)), _ptr(k_pages), _ptr(v_pages),
         c_int(_code(k_pages)), _ptr(block_table), c_int(block_table.shape[1]), _ptr(cu_q), _ptr(ctx_len),
         _ptr(seg_of_token), c_int(T), c_int(num_heads), c_int(Hk), c_int(D), c_int(page_size),
-        c_float(scale), c_int(window or 0), _stream()), "paged_attention_simple")
+        c_float(scale), c_int(window or 0), _ptr(sinks), _stream()), "paged_attention_simple")
     return out
 
 
@@ -274,7 +285,8 @@ def tiled_attention_available(q: torch.Tensor, k_pages: torch.Tensor, q_row_stri
 def paged_attention_tiled_f32(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pages: torch.Tensor,
                               v_pages: torch.Tensor, block_table: torch.Tensor, cu_q: torch.Tensor,
                               ctx_len: torch.Tensor, num_tokens: int, max_q_len: int, num_heads: int,
-                              scale: float, window: Optional[int], num_splits: int = 1) -> torch.Tensor:
+                              scale: float, window: Optional[int], num_splits: int = 1,
+                              sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """float32 attention: 64 rows (tokens x the query heads of a KV head) a workgroup share the keys
     and values of their KV head through LDS (fp32 arithmetic on the vector ALU).  `num_splits` > 1
     cuts the key range of every tile into that many parts across workgroups, merged by a second kernel
@@ -282,6 +294,7 @@ def paged_attention_tiled_f32(q: torch.Tensor, q_row_stride: int, out: torch.Ten
     The tables may describe a run of the step's segments only: `num_tokens` then counts the tokens up
     to the end of the last of them, and only their rows of `out` are written."""
     _dev(q, out, k_pages, v_pages, block_table, cu_q, ctx_len)
+    _check_sinks(sinks, num_heads)
     P, Hk, page_size, D = k_pages.shape
     _check(tiled_attention_available(q, k_pages, q_row_stride),
            f"paged_attention_tiled_f32 takes float32, head sizes 16..128 in steps of 16 and page sizes that are "
@@ -307,20 +320,22 @@ def paged_attention_tiled_f32(q: torch.Tensor, q_row_stride: int, out: torch.Ten
         _ptr(q), c_int(q_row_stride), _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
         c_int(block_table.shape[1]), _ptr(cu_q), _ptr(ctx_len), c_int(B), c_int(T), c_int(max_q_len),
         c_int(num_heads), c_int(Hk), c_int(D), c_int(page_size), c_float(scale), c_int(window or 0),
-        c_int(num_splits), _ptr(part_o), _ptr(part_ml), _stream()), "paged_attention_tiled_f32")
+        c_int(num_splits), _ptr(part_o), _ptr(part_ml), _ptr(sinks), _stream()), "paged_attention_tiled_f32")
     return out
 
 
 def paged_attention_decode_f32(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pages: torch.Tensor,
                                v_pages: torch.Tensor, block_table: torch.Tensor, cu_q: torch.Tensor,
                                ctx_len: torch.Tensor, num_heads: int, scale: float, window: Optional[int],
-                               num_splits: int = 1, first_token: int = 0) -> torch.Tensor:
+                               num_splits: int = 1, first_token: int = 0,
+                               sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """float32 attention of B segments of one token each, a run of the step's tokens that begins at
     token `first_token` (the tables may be a slice of a longer step's; cu_q[i] must be first_token + i,
     which the caller knows on the host and the kernels do not check): a wave takes up to four query
     heads of a KV head, so that the keys and values are read once for them.  `num_splits` > 1 cuts
     every key range into that many parts across workgroups, merged by a second kernel."""
     _dev(q, out, k_pages, v_pages, block_table, cu_q, ctx_len)
+    _check_sinks(sinks, num_heads)
     P, Hk, page_size, D = k_pages.shape
     _check(tiled_attention_available(q, k_pages, q_row_stride),
            f"paged_attention_decode_f32 takes float32, head sizes 16..128 in steps of 16 and page sizes that are "
@@ -349,7 +364,7 @@ def paged_attention_decode_f32(q: torch.Tensor, q_row_stride: int, out: torch.Te
         _ptr(q), c_int(q_row_stride), _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
         c_int(block_table.shape[1]), _ptr(cu_q), _ptr(ctx_len), c_int(B), c_int(first_token), c_int(num_heads),
         c_int(Hk), c_int(D), c_int(page_size), c_float(scale), c_int(window or 0), c_int(num_splits), _ptr(part_o),
-        _ptr(part_ml), _stream()), "paged_attention_decode_f32")
+        _ptr(part_ml), _ptr(sinks), _stream()), "paged_attention_decode_f32")
     return out
 
 
@@ -364,16 +379,28 @@ TILED_MIN_CONTEXT = 256
 FP32_DECODE_WAVES = 2048
 
 
-def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i]."""
+# gated activations (csrc/common.h, gate_mul): silu(g) u; gelu_tanh(g) u; and, with g' = min(g, limit) and
+# u' = clamp(u, -limit, limit), g' sigmoid(1.702 g') (u' + 1)
+GATES = {"silu": 0, "gelu_tanh": 1, "clamped_swish": 2}
+
+
+def gate_mul(gate_up: torch.Tensor, out: torch.Tensor, kind: str = "silu", limit: float = 0.0) -> torch.Tensor:
+    """out[t, i] = gate(gate_up[t, i], gate_up[t, I + i]) for one of GATES; fp32 arithmetic."""
     _dev(gate_up, out)
     T, two_i = gate_up.shape
+    _check(kind in GATES, f"unknown gate {kind!r}; known: {sorted(GATES)}")
+    _check(kind != "clamped_swish" or limit > 0.0, "the clamped gate needs a positive limit")
     _check(two_i % 2 == 0 and out.shape == (T, two_i // 2) and out.dtype == gate_up.dtype,
-           "silu_mul: out must be [T, I] for gate_up [T, 2 I]")
+           "gate_mul: out must be [T, I] for gate_up [T, 2 I]")
     lib = load_library("elementwise")
-    _ret(lib.sa_silu_mul(_ptr(gate_up), _ptr(out), c_int(_code(out)), c_int(T), c_int(two_i // 2), _stream()),
-         "silu_mul")
+    _ret(lib.sa_gate_mul(_ptr(gate_up), _ptr(out), c_int(_code(out)), c_int(T), c_int(two_i // 2),
+                         c_int(GATES[kind]), c_float(limit), _stream()), "gate_mul")
     return out
+
+
+def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i]."""
+    return gate_mul(gate_up, out, "silu")
 
 
 # ---------------------------------------------------------------------------------------------
@@ -527,12 +554,65 @@ def head_linear(x: torch.Tensor, in_stride: int, in_head_stride: int, w: torch.T
 
 
 # ---------------------------------------------------------------------------------------------
+# attention with normed queries and keys
+# ---------------------------------------------------------------------------------------------
+
+def qk_norm_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, positions: torch.Tensor, slots: Optional[torch.Tensor],
+                     k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor], q_weight: torch.Tensor,
+                     k_weight: torch.Tensor, eps: float, num_heads: int, num_kv_heads: int, dim: int, vdim: int,
+                     temp_coef: float = 0.0, temp_every: int = 0, v_first: Optional[torch.Tensor] = None,
+                     v_blend: float = 0.0) -> torch.Tensor:
+    """From rows qkv [T, Hq D | Hk D | Hk Dv]: every query and key head over its root mean square (eps inside
+    the root) times `q_weight` / `k_weight` (fp32 [D]); queries at position p times
+    1 + temp_coef * ln(floor((p + 1) / temp_every) + 1) (temp_every 0: not); values blended as
+    (1 - v_blend) v + v_blend v_first (v_first [T, >= Hk Dv] rows, may be a view with a row stride; None: not).
+    Queries go to q_out [T, Hq Dp], keys and values to the token's slot of k_pages [P, Hk, page, Dp] and
+    v_pages [P, Hk, Dp, page], each padded with zeros up to the cache's head size Dp.  `slots` None: queries only."""
+    _dev(q_out, positions, slots, k_pages, v_pages, q_weight, k_weight)
+    Hq, Hk, D, Dv = num_heads, num_kv_heads, dim, vdim
+    T = qkv.shape[0]
+    _check(qkv.is_cuda and qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] >= Hq * D + Hk * (D + Dv),
+           f"qkv must be rows of at least {Hq * D + Hk * (D + Dv)} on the GPU")
+    _check(q_out.dim() == 2 and q_out.shape[0] == T and q_out.shape[1] % Hq == 0 and q_out.dtype == qkv.dtype,
+           "q_out must be [T, Hq Dp] in the dtype of qkv")
+    Dp = q_out.shape[1] // Hq
+    _check(Dp >= D and Dp >= Dv, f"the padded head size {Dp} is below dim {D} or vdim {Dv}")
+    _f32vec(q_weight, D, "q norm weight")
+    _f32vec(k_weight, D, "k norm weight")
+    _i32(positions, T, "positions")
+    page_size = 1
+    if slots is not None:
+        _i32(slots, T, "slots")
+        P, _, page_size, _ = k_pages.shape
+        _check(k_pages.shape == (P, Hk, page_size, Dp) and v_pages.shape == (P, Hk, Dp, page_size),
+               f"the cache must be k [P, {Hk}, page, {Dp}] and v [P, {Hk}, {Dp}, page]")
+        _check(k_pages.dtype == qkv.dtype and v_pages.dtype == qkv.dtype, "cache dtype must match activations")
+    vf_stride = 0
+    if v_first is not None:
+        _check(v_first.is_cuda and v_first.device == qkv.device and v_first.dim() == 2 and v_first.shape[0] == T
+               and v_first.stride(1) == 1 and v_first.shape[1] >= Hk * Dv and v_first.dtype == qkv.dtype,
+               f"v_first must be [T, >= {Hk * Dv}] rows in the dtype of qkv")
+        vf_stride = v_first.stride(0)
+    _check(temp_every >= 0, "temp_every must not be negative")
+    lib = load_library("qk_norm")
+    _ret(lib.sa_qk_norm_kv_write(_ptr(qkv), c_int(qkv.stride(0)), _ptr(q_out), c_int(_code(qkv)), _ptr(positions),
+                                 _ptr(slots), _ptr(k_pages if slots is not None else None),
+                                 _ptr(v_pages if slots is not None else None), _ptr(q_weight), _ptr(k_weight),
+                                 c_float(eps), c_float(temp_coef), c_int(temp_every), _ptr(v_first), c_int(vf_stride),
+                                 c_float(v_blend), c_int(T), c_int(Hq), c_int(Hk), c_int(D), c_int(Dv), c_int(Dp),
+                                 c_int(page_size), _stream()), "qk_norm_kv_write")
+    return q_out
+
+
+# ---------------------------------------------------------------------------------------------
 # routed experts
 # ---------------------------------------------------------------------------------------------
 
-def moe_route(logits: torch.Tensor, experts: int, top: int, ids: torch.Tensor, weights: torch.Tensor) -> None:
+def moe_route(logits: torch.Tensor, experts: int, top: int, ids: torch.Tensor, weights: torch.Tensor,
+              over_all: bool = False, scale: float = 1.0) -> None:
     """Per row of logits fp32 [T, >= experts]: the `top` experts with the largest logits (ids int32
-    [T, top]) and the softmax over those logits alone (weights fp32 [T, top])."""
+    [T, top]) and their weights fp32 [T, top]: the softmax over those logits alone, or (`over_all`) their
+    shares of the softmax over all experts divided by the sum of the chosen shares + 1e-20; times `scale`."""
     _dev(logits, ids, weights)
     T = logits.shape[0]
     _check(logits.dtype == torch.float32 and logits.dim() == 2 and logits.shape[1] >= experts, "router logits must be fp32 [T, >= E]")
@@ -541,7 +621,7 @@ def moe_route(logits: torch.Tensor, experts: int, top: int, ids: torch.Tensor, w
            "ids int32 [T, top], weights fp32 [T, top]")
     lib = load_library("moe")
     _ret(lib.sa_moe_route(_ptr(logits), c_int(logits.shape[1]), _ptr(ids), _ptr(weights), c_int(T), c_int(experts),
-                          c_int(top), _stream()), "moe_route")
+                          c_int(top), c_int(1 if over_all else 0), c_float(scale), _stream()), "moe_route")
 
 
 MOE_ROUTE_INSIDE = 16      # up to this many tokens the experts' call does the routing itself (one kernel less)
@@ -549,10 +629,12 @@ MOE_ROUTE_INSIDE = 16      # up to this many tokens the experts' call does the r
 
 def moe_experts(h: torch.Tensor, ids: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor,
                 yk: torch.Tensor, logits: Optional[torch.Tensor] = None,
-                weights: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """yk[t * top + k] = expert ids[t, k] applied to h[t]: down(silu(gate h) * up h), fp32 [T top, d].
+                weights: Optional[torch.Tensor] = None, over_all: bool = False, scale: float = 1.0,
+                gate: str = "silu", limit: float = 0.0) -> torch.Tensor:
+    """yk[t * top + k] = expert ids[t, k] applied to h[t]: down(gate(gate h, up h)), fp32 [T top, d], with
+    one of GATES (silu(g) u unless said otherwise).
     w_gate, w_up [E, F, d], w_down [E, d, F] in h's dtype.  With `logits` (fp32 [T, >= E], at most
-    MOE_ROUTE_INSIDE tokens) `ids` and `weights` are made here as `moe_route` makes them."""
+    MOE_ROUTE_INSIDE tokens) `ids` and `weights` are made here as `moe_route` makes them (`over_all`, `scale`)."""
     _dev(h, ids, w_gate, w_up, w_down, yk, logits, weights)
     T, d = h.shape
     top = ids.shape[1]
@@ -561,6 +643,8 @@ def moe_experts(h: torch.Tensor, ids: torch.Tensor, w_gate: torch.Tensor, w_up: 
     _check(w_gate.dtype == h.dtype and w_up.dtype == h.dtype and w_down.dtype == h.dtype, "experts and activations must share a dtype")
     _check(ids.dtype == torch.int32 and ids.shape == (T, top), "ids must be int32 [T, top]")
     _check(yk.dtype == torch.float32 and yk.shape == (T * top, d), "yk must be fp32 [T top, d]")
+    _check(gate in GATES and (gate != "clamped_swish" or limit > 0.0), f"gate must be one of {sorted(GATES)}, "
+           "the clamped one with a positive limit")
     lib = load_library("moe")
     n = T * top
     tiles = int(lib.sa_moe_max_tiles(c_int(n), c_int(E)))
@@ -575,7 +659,8 @@ def moe_experts(h: torch.Tensor, ids: torch.Tensor, w_gate: torch.Tensor, w_up: 
         ldz = logits.shape[1]
     _ret(lib.sa_moe_experts(_ptr(h), c_int(_code(h)), _ptr(ids), _ptr(w_gate), _ptr(w_up), _ptr(w_down), _ptr(ints),
                             _ptr(act), _ptr(yk), c_int(T), c_int(top), c_int(E), c_int(d), c_int(F), _ptr(logits),
-                            c_int(ldz), _ptr(weights), _stream()), "moe_experts")
+                            c_int(ldz), _ptr(weights), c_int(1 if over_all else 0), c_float(scale), c_int(GATES[gate]),
+                            c_float(limit), _stream()), "moe_experts")
     return yk
 
 
@@ -899,13 +984,15 @@ def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, 
                          v_pages: torch.Tensor, block_table: torch.Tensor, cu_q: torch.Tensor,
                          ctx_len: torch.Tensor, num_tokens: int, max_q_len: int, num_heads: int, scale: float,
                          window: Optional[int], num_splits: int = 1, seg_begin: int = 0,
-                         seg_count: Optional[int] = None, in_workgroup: bool = False) -> torch.Tensor:
+                         seg_count: Optional[int] = None, in_workgroup: bool = False,
+                         sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """bf16 attention on the matrix cores (head sizes 16..128 in steps of 16, page sizes that are
     multiples of 4).  `in_workgroup` (segments of at most 16 rows per KV head, num_splits 1): the
     key range is cut four ways over the waves of a workgroup, which merges the parts itself.  `seg_begin`, `seg_count`: run only these segments of the step (their
     tokens' rows of `out` are written, the others left alone); `num_tokens` then is the number of
     tokens up to the end of the last of them."""
     _dev(q, out, k_pages, v_pages, block_table, cu_q, ctx_len)
+    _check_sinks(sinks, num_heads)
     P, Hk, page_size, D = k_pages.shape
     _check(mfma_attention_available(q, k_pages, q_row_stride, scale),
            f"paged_attention_mfma takes bf16, head sizes {MFMA_ATTENTION_HEAD_DIMS}, page sizes that are "
@@ -944,7 +1031,7 @@ def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, 
         _ptr(q), c_int(q_row_stride), _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
         c_int(block_table.shape[1]), _ptr(cu_q), _ptr(ctx_len), c_int(B), c_int(T), c_int(max_q_len),
         c_int(num_heads), c_int(Hk), c_int(D), c_int(page_size), c_float(scale), c_int(window or 0),
-        c_int(num_splits), _ptr(part_o), _ptr(part_ml), c_int(1 if in_workgroup else 0), _stream()),
+        c_int(num_splits), _ptr(part_o), _ptr(part_ml), c_int(1 if in_workgroup else 0), _ptr(sinks), _stream()),
         "paged_attention_mfma")
     return out
 
@@ -999,11 +1086,12 @@ def _attention_launches(ctx):
 
 def paged_attention(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pages: torch.Tensor,
                     v_pages: torch.Tensor, block_table: torch.Tensor, ctx, num_heads: int, scale: float,
-                    window: Optional[int]) -> torch.Tensor:
+                    window: Optional[int], sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention over the paged cache for all tokens of the step described by `ctx` (an `AttentionStep`,
     or anything with its attributes: the engine passes its `StepContext`): the matrix-core kernel for
     bf16 where it takes the sizes, else the general fp32-arithmetic kernel.  The plan of launches is
-    kept on `ctx`, so that the layers of a step share it."""
+    kept on `ctx`, so that the layers of a step share it.  `sinks` (fp32 [Hq]): one more term exp(sinks[h])
+    in the denominator of head h's softmax, in every kernel."""
     if mfma_attention_available(q, k_pages, q_row_stride, scale):
         Hk = k_pages.shape[1]
         # (first segment, segments, tokens up to their end, longest portion, longest context)
@@ -1014,7 +1102,8 @@ def paged_attention(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pag
             if not inside and (max_q == 1 or s0 == 0):
                 splits = attention_splits(max_q, n, Hk, max_ctx, num_heads // Hk)
             paged_attention_mfma(q, q_row_stride, out, k_pages, v_pages, block_table, ctx.cu_q, ctx.ctx_len,
-                                 t_end, max_q, num_heads, scale, window, splits, s0, n, in_workgroup=inside)
+                                 t_end, max_q, num_heads, scale, window, splits, s0, n, in_workgroup=inside,
+                                 sinks=sinks)
         return out
     Hk = k_pages.shape[1]
     if tiled_attention_available(q, k_pages, q_row_stride):
@@ -1034,14 +1123,14 @@ def paged_attention(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_pag
                     waves = n * Hk * -(-G // 4)
                     splits = max(1, min(64, FP32_DECODE_WAVES // max(waves, 1), max_ctx // 128))
                     paged_attention_decode_f32(q, q_row_stride, out, k_pages, v_pages, bt, cu, cl, num_heads, scale,
-                                               window, splits)
+                                               window, splits, sinks=sinks)
                     continue
                 splits = 1
                 if max_q * G <= TILED_MIN_ROWS and max_ctx >= TILED_MIN_CONTEXT and s0 == 0:
                     # few rows over many keys: about two workgroups per compute unit, parts of at least 256 keys
                     splits = max(1, min(64, 2 * compute_units() // max(n * Hk, 1), max_ctx // 256))
                 paged_attention_tiled_f32(q, q_row_stride, out, k_pages, v_pages, bt, cu, cl, t_end, max_q,
-                                          num_heads, scale, window, splits)
+                                          num_heads, scale, window, splits, sinks=sinks)
             return out
     return paged_attention_simple(q, q_row_stride, out, k_pages, v_pages, block_table, ctx.cu_q,
-                                  ctx.ctx_len, ctx.seg_of_token, ctx.num_tokens, num_heads, scale, window)
+                                  ctx.ctx_len, ctx.seg_of_token, ctx.num_tokens, num_heads, scale, window, sinks)

@@ -2,4 +2,4 @@
 from .base import (CacheTensor, LayerCache, ParamRequest, Part, PositionPart, Rotary, Runtime,  # noqa: F401
                    StateRequest, TokenCacheRequest, kv_cache_request)
 from . import standard  # noqa: F401
-from . import postnorm, recurrent, latent, feedforward  # noqa: F401
+from . import postnorm, recurrent, latent, feedforward, normed_attention  # noqa: F401

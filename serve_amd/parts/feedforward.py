@@ -43,18 +43,33 @@ class RoutedExperts(Part):
     with the largest router logits, weighted by the softmax over the chosen logits alone; the router's
     product gives fp32.  `shared_size`: one more expert of that width runs for every token and is added,
     times sigmoid(w_sg . x) if `shared_gate`.  The tokens are grouped by expert on the device; nothing is
-    read back, so steps with this part can be replayed from graphs."""
+    read back, so steps with this part can be replayed from graphs.
+
+    `activation` / `limit`: another gate of `ops.GATES` in the experts (`shared_limit`: the shared expert's
+    limit, if it differs).  `router_softmax="all"`: the weights are the chosen experts' shares of the softmax
+    over all experts, divided by their sum (+ 1e-20); `router_scale` multiplies the weights."""
 
     graph_safe = True
 
     def __init__(self, hidden_size: int, experts: int, top: int, expert_size: int,
-                 shared_size: Optional[int] = None, shared_gate: bool = True):
+                 shared_size: Optional[int] = None, shared_gate: bool = True, activation: str = "silu",
+                 limit: float = 0.0, shared_limit: Optional[float] = None, router_softmax: str = "chosen",
+                 router_scale: float = 1.0):
         if not 0 < top <= experts:
             raise ValueError("top must be within the number of experts")
+        if router_softmax not in ("chosen", "all"):
+            raise ValueError("router_softmax must be 'chosen' or 'all'")
+        if activation not in ops.GATES:
+            raise ValueError(f"unknown gate {activation!r}; known: {sorted(ops.GATES)}")
         self.hidden_size, self.experts, self.top, self.expert_size = int(hidden_size), int(experts), int(top), int(expert_size)
         self.shared_size = None if not shared_size else int(shared_size)
         self.shared_gate = bool(shared_gate) and self.shared_size is not None
-        self.shared = SwiGLU(self.hidden_size, self.shared_size) if self.shared_size else None
+        self.activation, self.limit = activation, float(limit)
+        self.over_all, self.router_scale = router_softmax == "all", float(router_scale)
+        self.shared = None
+        if self.shared_size:
+            self.shared = SwiGLU(self.hidden_size, self.shared_size, activation,
+                                 self.limit if shared_limit is None else float(shared_limit))
 
     def param_requests(self) -> List[ParamRequest]:
         d, F = self.hidden_size, self.expert_size
@@ -105,10 +120,11 @@ class RoutedExperts(Part):
         weights = torch.empty((T, self.top), dtype=torch.float32, device=dev)
         yk = torch.empty((T * self.top, d), dtype=torch.float32, device=dev)
         if T <= ops.MOE_ROUTE_INSIDE:
-            ops.moe_experts(h, ids, self.w_gate, self.w_up, self.w_down, yk, logits, weights)   # routes, too
+            ops.moe_experts(h, ids, self.w_gate, self.w_up, self.w_down, yk, logits, weights, self.over_all,
+                            self.router_scale, self.activation, self.limit)                    # routes, too
         else:
-            ops.moe_route(logits, self.experts, self.top, ids, weights)
-            ops.moe_experts(h, ids, self.w_gate, self.w_up, self.w_down, yk)
+            ops.moe_route(logits, self.experts, self.top, ids, weights, self.over_all, self.router_scale)
+            ops.moe_experts(h, ids, self.w_gate, self.w_up, self.w_down, yk, gate=self.activation, limit=self.limit)
         shared = self.shared.forward(h, ctx) if self.shared is not None else None
         y = torch.empty((T, d), dtype=torch.float32, device=dev)
         return ops.moe_combine(yk, weights, shared, logits if self.shared_gate else None, self.experts, y)

@@ -6,6 +6,12 @@ The sublayers read the residual stream itself (its copy in the activation dtype)
 weights may be stored around zero (`offset` 1), and every sublayer's normed output is scaled
 element by element (`scale`, a "layer scale") before it joins the stream.  A layer may have no
 feed-forward.
+
+And layers with a norm on both sides of every sublayer (`SandwichResidual`):
+
+    x <- x + c * Nb1(mixer(Na1(x)));   x <- x + c * Nb2(ffn(Na2(x)))
+
+with one constant c for the model in place of the layer scale.
 """
 from __future__ import annotations
 
@@ -24,17 +30,28 @@ class ScaledOutputNorm(Part):
 
     graph_safe = True
 
-    def __init__(self, size: int, eps: float, offset: float = 0.0):
+    def __init__(self, size: int, eps: float, offset: float = 0.0, constant_scale: Optional[float] = None):
+        """`constant_scale`: one number in place of the stored layer scale (no `scale` tensor then)."""
         self.size, self.eps, self.offset = int(size), float(eps), float(offset)
+        self.constant_scale = None if constant_scale is None else float(constant_scale)
 
     def param_requests(self) -> List[ParamRequest]:
-        return [ParamRequest("weight", (self.size,), init="normal:0.2" if self.offset else "ones_normal"),
-                ParamRequest("scale", (self.size,), init="ones_normal:0.2")]
+        out = [ParamRequest("weight", (self.size,), init="normal:0.2" if self.offset else "ones_normal")]
+        if self.constant_scale is None:
+            out.append(ParamRequest("scale", (self.size,), init="ones_normal:0.2"))
+        return out
 
     def load(self, tensors, rt: Runtime) -> None:
         self.rt = rt
         self.weight = (tensors["weight"].float() + self.offset).contiguous()       # fp32, whatever the storage
-        self.scale = tensors["scale"].float().contiguous()
+        if self.constant_scale is None:
+            self.scale = tensors["scale"].float().contiguous()
+        else:
+            self.scale = torch.full((self.size,), self.constant_scale, dtype=torch.float32, device=rt.device)
+
+    def add(self, x: torch.Tensor, y: torch.Tensor) -> None:
+        """Only x += scale * N(y): no copy of the stream is made."""
+        ops.output_norm_add(x, y, self.weight, self.scale, self.eps, None)
 
     def forward(self, x: torch.Tensor, y: Optional[torch.Tensor], rows=None) -> torch.Tensor:
         """Add the normed, scaled `y` into x (in place) and return what the next sublayer reads: x
@@ -94,5 +111,43 @@ class PostNormResidual:
         return None
 
 
+class SandwichResidual:
+    """x += c Nb1(mixer(Na1(x))); x += c Nb2(ffn(Na2(x))), the second half only if the layer has a feed-forward.
+
+    `mixer_norm` and `ffn_norm` are norms of the stream (kind `rmsnorm`), `mixer_out_norm` and `ffn_out_norm`
+    norms of a sublayer's output that add into the stream (kind `scaled_output_rmsnorm`, which carries c).
+    It leaves no pending output: the stream is complete when the layer returns."""
+
+    PART_ROLES = {"mixer": "mixer", "ffn": "feed_forward", "mixer_norm": "norm", "mixer_out_norm": "norm",
+                  "ffn_norm": "norm", "ffn_out_norm": "norm"}
+    OPTIONAL_PARTS = ("ffn", "ffn_norm", "ffn_out_norm")
+
+    def __init__(self, mixer, mixer_norm, mixer_out_norm, ffn=None, ffn_norm=None, ffn_out_norm=None):
+        if not ((ffn is None) == (ffn_norm is None) == (ffn_out_norm is None)):
+            raise ValueError("a feed-forward and its two norms come together")
+        self.mixer, self.mixer_norm, self.mixer_out_norm = mixer, mixer_norm, mixer_out_norm
+        self.ffn, self.ffn_norm, self.ffn_out_norm = ffn, ffn_norm, ffn_out_norm
+
+    def cache_owner(self) -> Part:
+        return self.mixer
+
+    def parts(self) -> Dict[str, Part]:
+        out = {"mixer": self.mixer, "mixer_norm": self.mixer_norm, "mixer_out_norm": self.mixer_out_norm}
+        if self.ffn is not None:
+            out.update(ffn=self.ffn, ffn_norm=self.ffn_norm, ffn_out_norm=self.ffn_out_norm)
+        return out
+
+    def forward(self, x: torch.Tensor, pending: Optional[torch.Tensor], ctx, cache: LayerCache,
+                writes_cache: bool = True) -> None:
+        ctx.stream_copy = None                      # (this layer changes the stream and keeps no such copy)
+        h = self.mixer_norm.forward(x, pending)     # (adds what a layer of another arrangement left unadded)
+        self.mixer_out_norm.add(x, self.mixer.forward(h, ctx, cache, writes_cache))
+        if self.ffn is not None:
+            h = self.ffn_norm.forward(x, None)
+            self.ffn_out_norm.add(x, self.ffn.forward(h, ctx))
+        return None
+
+
 register_part("norm", "scaled_output_rmsnorm", ScaledOutputNorm)
 register_part("arrangement", "postnorm_residual", PostNormResidual)
+register_part("arrangement", "sandwich_residual", SandwichResidual)

@@ -221,12 +221,18 @@ class GQAAttention(Part):
 # ---------------------------------------------------------------------------------------------
 class SwiGLU(Part):
     """down(silu(gate x) * up x), no biases (serve/model.py:71-85); gate and up run as one
-    product over the stacked matrix."""
+    product over the stacked matrix.  `activation` names another gate of `ops.GATES` in place of
+    silu(g) u: "gelu_tanh", or "clamped_swish" with its `limit`."""
 
     graph_safe = True
 
-    def __init__(self, hidden_size: int, intermediate_size: int):
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu", limit: float = 0.0):
+        if activation not in ops.GATES:
+            raise ValueError(f"unknown gate {activation!r}; known: {sorted(ops.GATES)}")
+        if activation == "clamped_swish" and not limit > 0.0:
+            raise ValueError("the clamped gate needs a positive limit")
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.activation, self.limit = activation, float(limit)
 
     def param_requests(self) -> List[ParamRequest]:
         d, i = self.hidden_size, self.intermediate_size
@@ -244,13 +250,14 @@ class SwiGLU(Part):
     def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
         a = self.rt.empty((h.shape[0], self.intermediate_size))
         M = h.shape[0]
-        if (h.dtype == torch.bfloat16 and self.w_gate_up.dtype == torch.bfloat16 and self.hidden_size % 8 == 0
+        if (self.activation == "silu" and h.dtype == torch.bfloat16 and self.w_gate_up.dtype == torch.bfloat16
+                and self.hidden_size % 8 == 0
                 and (M <= ops.SKINNY_MAX_ROWS or (M <= ops.WIDE_MAX_ROWS and ops.gemm_takes_wide(
                     M, self.intermediate_size, self.hidden_size, 1, swiglu=True)))):
             ops.swiglu_bf16(h, self.w_gate_up, a)          # product and gate in one kernel
         else:
             gu = linear(h, self.w_gate_up)
-            ops.silu_mul(gu, a)
+            ops.gate_mul(gu, a, self.activation, self.limit)
         return linear(a, self.w_down, partial_ok=True)     # the following norm adds the parts
 
 
@@ -262,8 +269,10 @@ class TokenEmbedding(Part):
 
     graph_safe = True
 
-    def __init__(self, vocab_size: int, hidden_size: int):
-        self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
+    def __init__(self, vocab_size: int, hidden_size: int, scale: float = 1.0):
+        """`scale` multiplies every row as it enters the stream (in fp32; the table itself, which an
+        output head may share, stays as stored)."""
+        self.vocab_size, self.hidden_size, self.scale = int(vocab_size), int(hidden_size), float(scale)
 
     def param_requests(self) -> List[ParamRequest]:
         return [ParamRequest("weight", (self.vocab_size, self.hidden_size))]
@@ -281,7 +290,7 @@ class TokenEmbedding(Part):
         """The rows of the step's tokens.  `ctx.src_row` / `ctx.prev_tokens` (when set): rows whose
         token was sampled on the device by an earlier step and never reached the host."""
         x = self.rt.empty((ctx.token_ids.numel(), self.hidden_size), torch.float32)
-        return ops.embed(self.weight, ctx.token_ids, x, ctx.src_row, ctx.prev_tokens)
+        return ops.embed(self.weight, ctx.token_ids, x, ctx.src_row, ctx.prev_tokens, self.scale)
 
 
 class LinearHead(Part):
@@ -350,6 +359,7 @@ register_part("norm", "rmsnorm", RMSNorm)
 register_part("position", "rope", RotaryPosition)
 register_part("mixer", "gqa_attention", GQAAttention)
 register_part("feed_forward", "swiglu", SwiGLU)
+register_part("feed_forward", "gated", SwiGLU)            # (the same part under the name of its general form)
 register_part("embedding", "token_embedding", TokenEmbedding)
 register_part("lm_head", "linear_head", LinearHead)
 register_part("arrangement", "prenorm_residual", PreNormResidual)

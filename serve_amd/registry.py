@@ -83,3 +83,4 @@ def _ensure_builtin() -> None:
         from . import parts  # noqa: F401  (registers the part kinds)
         from .models import llama  # noqa: F401  (registers LlamaForCausalLM)
         from .models import zozosun  # noqa: F401  (registers Zozosun)
+        from .models import timopel  # noqa: F401  (registers Timopel)

@@ -473,7 +473,7 @@ def test_traces_through_the_program(tmp_path, dtype):
     import subprocess
     import numpy as np
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    name = "TB"
+    name = "TA"
     folder = tm.make_folder(tmp_path, name)
     vocab = tm.MODELS[name][0].vocab
     reqs, steps = {}, []

@@ -79,7 +79,31 @@ SHAPES.update({
     "llama-4k": LlamaConfig(vocab_size=32768, hidden_size=4096, intermediate_size=14336, num_hidden_layers=4,
                             num_attention_heads=32, num_key_value_heads=8, head_dim=128, rope_theta=500000.0),
 })
-DESIGN_PAIRS = (("zozosun-2k", "llama-2k"), ("zozosun-4k", "llama-4k"))
+
+
+def _timopel_shape(width: int, vocab: int, layers: int, heads: int, kv_heads: int, head: int, ff: int, experts: int,
+                   top: int, expert_ff: int, shared_ff: int):
+    """A Timopel shape at the sizes of a real model's layers: attention layers with `heads` on `kv_heads` heads of
+    `head` (keys and values alike), whose feed-forwards are in turn dense and routed experts with a shared one; all
+    layers but the first blend their values with the first layer's."""
+    from .config.timopel import (ClampedMoeConfig, GatedDenseConfig, QueryTemperature, SinkAttentionConfig,
+                                 TimopelConfig, TimopelLayerConfig)
+    mixer = SinkAttentionConfig(heads, kv_heads, head, head, head ** -0.5, QueryTemperature(0.1, 1024), True)
+    moe = ClampedMoeConfig(experts, top, 1.0, expert_ff, 7.0, shared_ff, 7.0)
+    return TimopelConfig(vocab=vocab, width=width, eps=1e-5, residual_mult=0.5, embedding_scale=1.0,
+                         layers=tuple(TimopelLayerConfig(mixer, GatedDenseConfig(ff) if i % 2 == 0 else moe)
+                                      for i in range(layers)))
+
+
+# Timopel at the same two widths, depths, vocabularies, head shapes and dense feed-forward widths as the Llama
+# shapes above (its experts as Zozosun's)
+SHAPES.update({
+    "timopel-tiny": _timopel_shape(64, 512, 2, 4, 2, 16, 128, 4, 2, 32, 64),
+    "timopel-2k": _timopel_shape(2048, 32768, 8, 32, 8, 64, 8192, 32, 4, 1024, 2048),
+    "timopel-4k": _timopel_shape(4096, 32768, 4, 32, 8, 128, 14336, 64, 6, 1536, 3072),
+})
+DESIGN_PAIRS = (("zozosun-2k", "llama-2k"), ("zozosun-4k", "llama-4k"), ("timopel-2k", "llama-2k"),
+                ("timopel-4k", "llama-4k"))
 
 
 def generate_requests(input_length: int, output_length: int, num_sequences: int, vocab_size: int,

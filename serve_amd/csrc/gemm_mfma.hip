@@ -32,7 +32,7 @@ union Frag {
 // gridDim.z > 1 cuts K across workgroups as well: workgroup z writes its partial sums to
 // C + z * M * N (fp32), and the consumer adds the parts in order.
 // EPI selects what is done with the sums: EPI_PLAIN stores them; EPI_SWIGLU pairs gate row n with up
-// row I + n and stores silu(gate) * up; EPI_QKV_ROPE works on one tile of 16 rows of the stacked
+// row I + n and stores silu(gate) * up (or another gate of common.h); EPI_QKV_ROPE works on one tile of 16 rows of the stacked
 // q/k/v matrix that holds eight dims j.. of a head and their partners j + D/2..: the sums of a pair
 // sit in lanes 32 apart and are exchanged with one row swap each, the q and k pairs are rotated by
 // position (the rotation of serve/model.py:234-244 on the checkpoint's row order), q goes to its
@@ -47,7 +47,17 @@ struct QkvRopeArgs {
   bf16_t* k_pages;          // [P, Hk, page_size, D]
   bf16_t* v_pages;          // [P, Hk, D, page_size]
   int Hq, Hk, D, page_size;
+  // the gate of the EPI_SWIGLU epilogue, one of common.h's (0 = silu(g) u), and the clamped gate's limit
+  int gate_kind;
+  float gate_limit;
 };
+
+// silu(g) u with the fast exponential, as the plain SwiGLU feed-forward has always been computed; any other gate
+// through gate_mul
+__device__ __forceinline__ float gated(float gt, float up, const QkvRopeArgs& qa) {
+  if (qa.gate_kind == SA_GATE_SILU) return (gt / (1.f + __expf(-gt))) * up;
+  return gate_mul(gt, up, qa.gate_kind, qa.gate_limit);
+}
 
 // What the rotating epilogue needs besides the sums: read when a kernel starts, so that the trip to
 // memory for them runs beside the product and not after it.
@@ -117,7 +127,7 @@ __device__ __forceinline__ void store_tiles(floatx4_t (&acc)[RT][MT], TC* __rest
       for (int r = 0; r < 4; ++r) {
         const float gt = acc[0][mt][r];
         const float up = acc[1][mt][r];
-        o[r] = (gt / (1.f + __expf(-gt))) * up;
+        o[r] = gated(gt, up, qa);
       }
       if (n + 3 < N) {
         store4(C + (size_t)m * ldc + n, o, (N & 3) == 0);
@@ -734,7 +744,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16_t* __restrict
       for (int r = 0; r < 4; ++r) {
         if (SWIGLU) {
           const float gt = acc[mt][nt][r];
-          o[r] = (gt / (1.f + __expf(-gt))) * acc[mt][SWIGLU ? nt + NT / 2 : nt][r];
+          o[r] = gated(gt, acc[mt][SWIGLU ? nt + NT / 2 : nt][r], qa);
         } else {
           o[r] = acc[mt][nt][r];
         }
@@ -1044,10 +1054,12 @@ extern "C" int sa_gemm_bf16_skinny(const void* A, const void* W, void* C, int c_
 
 // C[M, I] = silu(A Wg^T) * (A Wu^T) with W = [Wg; Wu] stacked as [2 I, K]
 extern "C" int sa_gemm_bf16_skinny_swiglu(const void* A, const void* W, void* C, int M, int I, int K,
-                                          hipStream_t stream) {
+                                          int gate_kind, float gate_limit, hipStream_t stream) {
   if (M <= 0 || I <= 0) return 0;
-  if (K <= 0 || (K & 7)) return SA_ERR_ARG;
-  const QkvRopeArgs none = {};
+  if (K <= 0 || (K & 7) || gate_kind < 0 || gate_kind >= SA_GATE_KINDS) return SA_ERR_ARG;
+  QkvRopeArgs none = {};
+  none.gate_kind = gate_kind;
+  none.gate_limit = gate_limit;
   if (takes_wide<bf16_t, EPI_SWIGLU>(M, I, K, 1)) return pick_wide<bf16_t, EPI_SWIGLU>(A, W, C, M, I, K, I, 1, none, stream);
   if (!takes_skinny<bf16_t, EPI_SWIGLU>(M, I, none)) return pick_mid<bf16_t, EPI_SWIGLU>(A, W, C, M, I, K, I, 1, none, stream);
   return pick_skinny<bf16_t, EPI_SWIGLU>(A, W, C, M, I, K, I, 1, none, stream);

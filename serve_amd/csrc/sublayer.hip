@@ -9,6 +9,9 @@
 // the stream next.  y is [T, d] in the activation dtype or fp32, or fp32 [parts, T, d] partial
 // sums that are added in order (a product whose inner dimension was cut across workgroups, the
 // experts of a token).  y == nullptr: only the copy h = x is made.  h == nullptr: no copy.
+// nw != nullptr (with y and h): h[t] = N(x[t]) * nw instead, the norm (eps `neps`) of the new stream that the
+// next sublayer reads: a layer with a norm behind one sublayer and another in front of the next needs one
+// kernel between the two.
 // One workgroup a row; a thread keeps up to VMAX of its values between the two passes, the rest
 // is read again.
 // ---------------------------------------------------------------------------------------------
@@ -17,7 +20,8 @@ __global__ __launch_bounds__(256) void output_norm_add_kernel(float* __restrict_
                                                               int parts, size_t part_stride,
                                                               const float* __restrict__ w,
                                                               const float* __restrict__ s, TA* __restrict__ h,
-                                                              float eps, int d) {
+                                                              float eps, int d, const float* __restrict__ nw,
+                                                              float neps) {
   __shared__ float scratch[16];
   constexpr int VMAX = 8;
   const int t = blockIdx.x;
@@ -48,13 +52,17 @@ __global__ __launch_bounds__(256) void output_norm_add_kernel(float* __restrict_
   }
   ss = block_sum(ss, scratch);
   const float rs = 1.0f / sqrtf(ss / (float)d + eps);
+  const bool copy = hr && !nw;
+  float ss2 = 0.f;
 #pragma unroll
   for (int n = 0; n < VMAX; ++n) {
     const int i = threadIdx.x + n * bd;
     if (i < d) {
       const float nx = xr[i] + ((keep[n] * rs) * w[i]) * s[i];
       xr[i] = nx;
-      if (hr) hr[i] = from_float<TA>(nx);
+      keep[n] = nx;
+      ss2 += nx * nx;
+      if (copy) hr[i] = from_float<TA>(nx);
     }
   }
   for (int i = threadIdx.x + VMAX * bd; i < d; i += bd) {
@@ -62,8 +70,19 @@ __global__ __launch_bounds__(256) void output_norm_add_kernel(float* __restrict_
     for (int p = 0; p < parts; ++p) v += to_float(yr[p * part_stride + i]);
     const float nx = xr[i] + ((v * rs) * w[i]) * s[i];
     xr[i] = nx;
-    if (hr) hr[i] = from_float<TA>(nx);
+    ss2 += nx * nx;
+    if (copy) hr[i] = from_float<TA>(nx);
   }
+  if (!hr || !nw) return;
+  // the norm of the new stream (every thread reads back only what it wrote itself)
+  ss2 = block_sum(ss2, scratch);
+  const float rs2 = rsqrtf(ss2 / (float)d + neps);
+#pragma unroll
+  for (int n = 0; n < VMAX; ++n) {
+    const int i = threadIdx.x + n * bd;
+    if (i < d) hr[i] = from_float<TA>((keep[n] * rs2) * nw[i]);
+  }
+  for (int i = threadIdx.x + VMAX * bd; i < d; i += bd) hr[i] = from_float<TA>((xr[i] * rs2) * nw[i]);
 }
 
 // The same for d % 4 == 0 and d <= 8192: 16-byte vectors, and every load of a row (the parts of y, x, w, s) is
@@ -88,7 +107,8 @@ __global__ __launch_bounds__(256) void output_norm_add_vec_kernel(float* __restr
                                                                   int parts, size_t part_stride,
                                                                   const float* __restrict__ w,
                                                                   const float* __restrict__ s, TA* __restrict__ h,
-                                                                  float eps, int d) {
+                                                                  float eps, int d, const float* __restrict__ nw,
+                                                                  float neps) {
   __shared__ float scratch[16];
   const int t = blockIdx.x;
   float* xr = x + (size_t)t * d;
@@ -129,15 +149,38 @@ __global__ __launch_bounds__(256) void output_norm_add_vec_kernel(float* __restr
       nx.z = xv[k].z + ((v[k].z * rs) * wv[k].z) * sv[k].z;
       nx.w = xv[k].w + ((v[k].w * rs) * wv[k].w) * sv[k].w;
       st4(xr + i, nx);
-      if (h) st4(h + (size_t)t * d + i, nx);
+      if (h && !nw) st4(h + (size_t)t * d + i, nx);
+      v[k] = nx;
+    }
+  }
+  if (!h || !nw) return;
+  // the norm of the new stream, from the values still in registers
+  float ss2 = 0.f;
+#pragma unroll
+  for (int k = 0; k < NG; ++k) {
+    const float in = threadIdx.x + k * 256 < groups ? 1.f : 0.f;
+    ss2 += in * (v[k].x * v[k].x + v[k].y * v[k].y + v[k].z * v[k].z + v[k].w * v[k].w);
+  }
+  ss2 = block_sum(ss2, scratch);
+  const float rs2 = rsqrtf(ss2 / (float)d + neps);
+#pragma unroll
+  for (int k = 0; k < NG; ++k) {
+    const int gi = threadIdx.x + k * 256;
+    if (gi < groups) {
+      const int i = gi * 4;
+      const float4 n4 = ld4(nw + i);
+      st4(h + (size_t)t * d + i, make_float4((v[k].x * rs2) * n4.x, (v[k].y * rs2) * n4.y, (v[k].z * rs2) * n4.z,
+                                             (v[k].w * rs2) * n4.w));
     }
   }
 }
 
 extern "C" int sa_output_norm_add(float* x, const void* y, int y_dtype, int parts, const float* w, const float* s,
-                                  void* h, int act_dtype, float eps, int T, int d, hipStream_t stream) {
+                                  void* h, int act_dtype, float eps, int T, int d, const float* nw, float neps,
+                                  hipStream_t stream) {
   if (T <= 0) return 0;
   if (d <= 0 || parts < 1) return SA_ERR_ARG;
+  if (nw && (!y || !h)) return SA_ERR_ARG;
   if (y && (!w || !s)) return SA_ERR_ARG;
   if (y && y_dtype != act_dtype && y_dtype != SA_F32) return SA_ERR_UNSUPPORTED;
   if (y && parts > 1 && y_dtype != SA_F32) return SA_ERR_UNSUPPORTED;
@@ -147,7 +190,7 @@ extern "C" int sa_output_norm_add(float* x, const void* y, int y_dtype, int part
     const int ng = (d / 4 + 255) / 256;          // groups of four a thread, 1 .. 8
 #define GOV(TA, TD, PMAX, NG)                                                                                   \
   hipLaunchKernelGGL((output_norm_add_vec_kernel<TA, TD, PMAX, NG>), grid, dim3(256), 0, stream, x,             \
-                     (const TD*)y, parts, part_stride, w, s, (TA*)h, eps, d)
+                     (const TD*)y, parts, part_stride, w, s, (TA*)h, eps, d, nw, neps)
 #define GON(TA, TD, PMAX)                                                                                       \
   do {                                                                                                          \
     if (ng <= 1) GOV(TA, TD, PMAX, 1);                                                                          \
@@ -172,7 +215,7 @@ extern "C" int sa_output_norm_add(float* x, const void* y, int y_dtype, int part
   }
 #define GO(TA, TD)                                                                                          \
   hipLaunchKernelGGL((output_norm_add_kernel<TA, TD>), grid, block, 0, stream, x, (const TD*)y, parts,      \
-                     part_stride, w, s, (TA*)h, eps, d)
+                     part_stride, w, s, (TA*)h, eps, d, nw, neps)
   const bool yfloat = !y || y_dtype == SA_F32;
   if (act_dtype == SA_F32) GO(float, float);
   else if (act_dtype == SA_BF16) { if (yfloat) GO(bf16_t, float); else GO(bf16_t, bf16_t); }

@@ -82,6 +82,8 @@ class StepContext:
     # layers blend with theirs, a normed stream made ahead for the layer that reads it); emptied by the model
     # at the start of a step
     shared: dict = field(default_factory=dict)
+    # the norm that the next layer of the run order begins with (None: unknown, or the layer does not say)
+    next_input_norm: object = None
 
 
 def _align(n: int) -> int:

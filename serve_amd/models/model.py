@@ -168,7 +168,12 @@ class Model:
         ctx.stream_copy = None          # (what a layer may leave for the next: the stream in the activation dtype)
         ctx.shared = {}                 # (and what layers leave for later layers of the step, by name)
         pending = None
-        for e in self.spec.run_order:
+        order = self.spec.run_order
+        for i, e in enumerate(order):
+            # the norm the next layer begins with, where its arrangement says so: this layer may apply it at the
+            # end of its own last kernel and leave the result in ctx.shared
+            nxt = self.layers[order[i + 1].layer] if i + 1 < len(order) else None
+            ctx.next_input_norm = nxt.input_norm() if hasattr(nxt, "input_norm") else None
             pending = self.layers[e.layer].forward(x, pending, ctx, caches[e.cache], e.writes_cache)
         if ctx.num_logit_rows == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=x.device)

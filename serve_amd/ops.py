@@ -412,11 +412,14 @@ def _f32vec(t: torch.Tensor, n: int, name: str) -> None:
 
 
 def output_norm_add(x: torch.Tensor, y: Optional[torch.Tensor], weight: Optional[torch.Tensor],
-                    scale: Optional[torch.Tensor], eps: float, h: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+                    scale: Optional[torch.Tensor], eps: float, h: Optional[torch.Tensor],
+                    next_weight: Optional[torch.Tensor] = None, next_eps: float = 0.0) -> Optional[torch.Tensor]:
     """x += (y / sqrt(mean(y^2) + eps) * weight) * scale on the fp32 residual stream x [T, d], in place;
     `h` (activation dtype [T, d]) receives a copy of the new x.  y is [T, d] in h's dtype or fp32, or
-    fp32 [parts, T, d] partial sums that are added in order.  y None: only the copy is made."""
-    _dev(x, y, weight, scale, h)
+    fp32 [parts, T, d] partial sums that are added in order.  y None: only the copy is made.
+    With `next_weight` (fp32 [d]; needs y and h): h = x / sqrt(mean(x^2) + next_eps) * next_weight of the new
+    x instead of its copy: the norm in front of the sublayer that reads the stream next."""
+    _dev(x, y, weight, scale, h, next_weight)
     _check(x.dtype == torch.float32 and x.dim() == 2, "residual stream must be fp32 [T, d]")
     T, d = x.shape
     act = h.dtype if h is not None else (y.dtype if y is not None and y.dim() == 2 else torch.float32)
@@ -432,9 +435,13 @@ def output_norm_add(x: torch.Tensor, y: Optional[torch.Tensor], weight: Optional
         ycode = _code(y)
     if h is not None:
         _check(h.shape == (T, d), "the stream's copy must be [T, d]")
+    if next_weight is not None:
+        _check(y is not None and h is not None, "the norm of the new stream needs a sublayer's output and a place to go")
+        _f32vec(next_weight, d, "the next norm's weight")
     lib = load_library("sublayer")
     _ret(lib.sa_output_norm_add(_ptr(x), _ptr(y), c_int(ycode), c_int(parts), _ptr(weight), _ptr(scale), _ptr(h),
-                                c_int(_DT[act]), c_float(eps), c_int(T), c_int(d), _stream()), "output_norm_add")
+                                c_int(_DT[act]), c_float(eps), c_int(T), c_int(d), _ptr(next_weight), c_float(next_eps),
+                                _stream()), "output_norm_add")
     return h
 
 
@@ -867,9 +874,13 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tens
     return gemm_bf16_library(a, w, out)
 
 
-def swiglu_bf16(a: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """out[M, I] = silu(a @ Wg^T) * (a @ Wu^T) for w_gate_up = [Wg; Wu] ([2 I, K]), one kernel."""
+def swiglu_bf16(a: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, gate: str = "silu",
+                limit: float = 0.0) -> torch.Tensor:
+    """out[M, I] = silu(a @ Wg^T) * (a @ Wu^T) for w_gate_up = [Wg; Wu] ([2 I, K]), one kernel; or with another
+    of GATES in place of silu(g) u."""
     _dev(a, w_gate_up, out)
+    _check(gate in GATES and (gate != "clamped_swish" or limit > 0.0), f"gate must be one of {sorted(GATES)}, "
+           "the clamped one with a positive limit")
     M, K = a.shape
     I = w_gate_up.shape[0] // 2
     _check(w_gate_up.shape == (2 * I, K) and out.shape == (M, I), "swiglu_bf16: shapes do not match")
@@ -877,7 +888,7 @@ def swiglu_bf16(a: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor) -> 
            and K % 8 == 0 and _aligned16(a, w_gate_up, out), "swiglu_bf16 needs bf16 operands and K % 8 == 0")
     lib = load_library("gemm_mfma")
     _ret(lib.sa_gemm_bf16_skinny_swiglu(_ptr(a), _ptr(w_gate_up), _ptr(out), c_int(M), c_int(I), c_int(K),
-                                        _stream()), "swiglu_bf16")
+                                        c_int(GATES[gate]), c_float(limit), _stream()), "swiglu_bf16")
     return out
 
 

@@ -53,6 +53,12 @@ class ScaledOutputNorm(Part):
         """Only x += scale * N(y): no copy of the stream is made."""
         ops.output_norm_add(x, y, self.weight, self.scale, self.eps, None)
 
+    def add_then_norm(self, x: torch.Tensor, y: torch.Tensor, following) -> torch.Tensor:
+        """x += scale * N(y), and in the same kernel what the norm `following` (an `RMSNorm`) makes of the new
+        x: the activations that the next sublayer reads."""
+        h = self.rt.empty(tuple(x.shape))
+        return ops.output_norm_add(x, y, self.weight, self.scale, self.eps, h, following.weight_f32, following.eps)
+
     def forward(self, x: torch.Tensor, y: Optional[torch.Tensor], rows=None) -> torch.Tensor:
         """Add the normed, scaled `y` into x (in place) and return what the next sublayer reads: x
         itself in the float32 engine, else its copy in the activation dtype."""
@@ -111,12 +117,17 @@ class PostNormResidual:
         return None
 
 
+NORMED_STREAM = "normed_stream"     # (activations, the norm that made them) from one layer for the next, on the step's context
+
+
 class SandwichResidual:
     """x += c Nb1(mixer(Na1(x))); x += c Nb2(ffn(Na2(x))), the second half only if the layer has a feed-forward.
 
     `mixer_norm` and `ffn_norm` are norms of the stream (kind `rmsnorm`), `mixer_out_norm` and `ffn_out_norm`
     norms of a sublayer's output that add into the stream (kind `scaled_output_rmsnorm`, which carries c).
-    It leaves no pending output: the stream is complete when the layer returns."""
+    It leaves no pending output: the stream is complete when the layer returns.  Each norm behind a sublayer and the
+    norm in front of the next one are one kernel, across layers too: where the model says which norm the next layer
+    begins with (`ctx.next_input_norm`), the activations it makes travel on the step's context."""
 
     PART_ROLES = {"mixer": "mixer", "ffn": "feed_forward", "mixer_norm": "norm", "mixer_out_norm": "norm",
                   "ffn_norm": "norm", "ffn_out_norm": "norm"}
@@ -137,14 +148,27 @@ class SandwichResidual:
             out.update(ffn=self.ffn, ffn_norm=self.ffn_norm, ffn_out_norm=self.ffn_out_norm)
         return out
 
+    def input_norm(self) -> Part:
+        """The norm this layer begins with: the layer before may apply it at the end of its own last kernel."""
+        return self.mixer_norm
+
     def forward(self, x: torch.Tensor, pending: Optional[torch.Tensor], ctx, cache: LayerCache,
                 writes_cache: bool = True) -> None:
         ctx.stream_copy = None                      # (this layer changes the stream and keeps no such copy)
-        h = self.mixer_norm.forward(x, pending)     # (adds what a layer of another arrangement left unadded)
-        self.mixer_out_norm.add(x, self.mixer.forward(h, ctx, cache, writes_cache))
+        ready = ctx.shared.pop(NORMED_STREAM, None)
+        if ready is not None and ready[1] is self.mixer_norm and pending is None:
+            h = ready[0]                            # the layer before has made it, with this layer's norm
+        else:
+            h = self.mixer_norm.forward(x, pending)     # (adds what a layer of another arrangement left unadded)
+        y, last = self.mixer.forward(h, ctx, cache, writes_cache), self.mixer_out_norm
         if self.ffn is not None:
-            h = self.ffn_norm.forward(x, None)
-            self.ffn_out_norm.add(x, self.ffn.forward(h, ctx))
+            h = last.add_then_norm(x, y, self.ffn_norm)
+            y, last = self.ffn.forward(h, ctx), self.ffn_out_norm
+        following = getattr(ctx, "next_input_norm", None)
+        if getattr(following, "weight_f32", None) is not None and following.size == last.size:
+            ctx.shared[NORMED_STREAM] = (last.add_then_norm(x, y, following), following)
+        else:
+            last.add(x, y)
         return None
 
 

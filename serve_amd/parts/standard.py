@@ -46,6 +46,8 @@ class RMSNorm(Part):
         self.weight = tensors["weight"]
         if self.offset:
             self.weight = self.weight.float() + self.offset
+        # (for kernels that apply this norm at the end of another kernel's work and take fp32 vectors)
+        self.weight_f32 = self.weight if self.weight.dtype == torch.float32 else self.weight.float()
 
     def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor],
                 rows: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -250,11 +252,11 @@ class SwiGLU(Part):
     def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
         a = self.rt.empty((h.shape[0], self.intermediate_size))
         M = h.shape[0]
-        if (self.activation == "silu" and h.dtype == torch.bfloat16 and self.w_gate_up.dtype == torch.bfloat16
+        if (h.dtype == torch.bfloat16 and self.w_gate_up.dtype == torch.bfloat16
                 and self.hidden_size % 8 == 0
                 and (M <= ops.SKINNY_MAX_ROWS or (M <= ops.WIDE_MAX_ROWS and ops.gemm_takes_wide(
                     M, self.intermediate_size, self.hidden_size, 1, swiglu=True)))):
-            ops.swiglu_bf16(h, self.w_gate_up, a)          # product and gate in one kernel
+            ops.swiglu_bf16(h, self.w_gate_up, a, self.activation, self.limit)          # product and gate in one kernel
         else:
             gu = linear(h, self.w_gate_up)
             ops.gate_mul(gu, a, self.activation, self.limit)

@@ -12,8 +12,17 @@
 //
 // Input rows are [Hq D | Hk D | Hk Dv] (one product); q_out [T, Hq Dp]; k pages [P, Hk, page_size, Dp],
 // v pages [P, Hk, Dp, page_size]; slot[t] = page * page_size + offset, < 0: nothing stored.
-// One workgroup a token; a wave takes a head at a time (q heads, then k heads, then v heads).
+//
+// Two kernels: the general one (any sizes and alignments: a wave per (token, head), a lane an element at a time),
+// and one for sizes that are multiples of 8 from aligned rows, which moves 8 elements a lane (16 bytes of bf16):
+// its first blocks take the query and key heads, a group of lanes per head; its last blocks take the values with
+// neighbouring lanes on neighbouring tokens, so that the writes into the transposed value pages, where the
+// tokens of a page lie side by side, fall into common lines.
 #include "common.h"
+
+__device__ __forceinline__ float query_temp(const int* positions, int t, float coef, int every) {
+  return every > 0 ? 1.f + coef * logf((float)((positions[t] + 1) / every) + 1.f) : 1.f;
+}
 
 template <typename TA>
 __global__ __launch_bounds__(256) void qk_norm_kv_write_kernel(
@@ -23,59 +32,191 @@ __global__ __launch_bounds__(256) void qk_norm_kv_write_kernel(
     int v_first_stride, float lambda, int Hq, int Hk, int D, int Dv, int Dp, int page_size) {
   const int t = blockIdx.x;
   const int lane = threadIdx.x & (SA_WAVE - 1);
-  const int wave = threadIdx.x / SA_WAVE;
-  const int waves = blockDim.x / SA_WAVE;
+  const int u = blockIdx.y * (blockDim.x / SA_WAVE) + threadIdx.x / SA_WAVE;      // the head this wave takes
+  if (u >= Hq + 2 * Hk) return;
   const TA* row = qkv + (size_t)t * row_stride;
   const int s = slot ? slot[t] : -1;
   const int page = s >= 0 ? s / page_size : 0;
   const int off = s >= 0 ? s - page * page_size : 0;
-  float temp = 1.f;
-  if (temp_every > 0) temp = 1.f + temp_coef * logf((float)((positions[t] + 1) / temp_every) + 1.f);
   const TA zero = from_float<TA>(0.f);
+  if (u < Hq + Hk) {
+    // a query or a key head: norm over its D dims
+    const bool is_q = u < Hq;
+    const int g = is_q ? u : u - Hq;
+    if (!is_q && s < 0) return;
+    const TA* x = row + (size_t)u * D;
+    float ss = 0.f;
+    for (int i = lane; i < D; i += SA_WAVE) {
+      const float v = to_float(x[i]);
+      ss += v * v;
+    }
+    ss = wave_sum(ss);
+    const float rs = 1.0f / sqrtf(ss / (float)D + eps);
+    const float temp = is_q ? query_temp(positions, t, temp_coef, temp_every) : 1.f;
+    const float* w = is_q ? wq : wk;
+    TA* dst = is_q ? q_out + ((size_t)t * Hq + g) * Dp : k_pages + (((size_t)page * Hk + g) * page_size + off) * Dp;
+    for (int i = lane; i < Dp; i += SA_WAVE) {
+      TA o = zero;
+      if (i < D) {
+        float v = (to_float(x[i]) * rs) * w[i];
+        if (is_q) v *= temp;
+        o = from_float<TA>(v);
+      }
+      dst[i] = o;
+    }
+    return;
+  }
+  if (s < 0) return;
+  const int g = u - Hq - Hk;
+  const TA* x = row + (size_t)(Hq + Hk) * D + (size_t)g * Dv;
+  const TA* f = v_first ? v_first + (size_t)t * v_first_stride + (size_t)g * Dv : nullptr;
+  TA* dst = v_pages + ((size_t)page * Hk + g) * (size_t)Dp * page_size + off;
+  for (int i = lane; i < Dp; i += SA_WAVE) {
+    TA o = zero;
+    if (i < Dv) {
+      float v = to_float(x[i]);
+      if (f) v = (1.f - lambda) * v + lambda * to_float(f[i]);
+      o = from_float<TA>(v);
+    }
+    dst[(size_t)i * page_size] = o;
+  }
+}
 
-  for (int u = wave; u < Hq + 2 * Hk; u += waves) {
-    if (u < Hq + Hk) {
-      // a query or a key head: norm over its D dims
-      const bool is_q = u < Hq;
-      const int g = is_q ? u : u - Hq;
-      if (!is_q && s < 0) continue;
-      const TA* x = row + (size_t)u * D;
-      float ss = 0.f;
-      for (int i = lane; i < D; i += SA_WAVE) {
-        const float v = to_float(x[i]);
-        ss += v * v;
-      }
-      ss = wave_sum(ss);
-      const float rs = 1.0f / sqrtf(ss / (float)D + eps);
-      const float* w = is_q ? wq : wk;
-      TA* dst = is_q ? q_out + ((size_t)t * Hq + g) * Dp
-                     : k_pages + (((size_t)page * Hk + g) * page_size + off) * Dp;
-      for (int i = lane; i < Dp; i += SA_WAVE) {
-        TA o = zero;
-        if (i < D) {
-          float v = (to_float(x[i]) * rs) * w[i];
-          if (is_q) v *= temp;
-          o = from_float<TA>(v);
-        }
-        dst[i] = o;
-      }
-    } else {
-      if (s < 0) continue;
-      const int g = u - Hq - Hk;
-      const TA* x = row + (size_t)(Hq + Hk) * D + (size_t)g * Dv;
-      const TA* f = v_first ? v_first + (size_t)t * v_first_stride + (size_t)g * Dv : nullptr;
-      TA* dst = v_pages + ((size_t)page * Hk + g) * (size_t)Dp * page_size + off;
-      for (int i = lane; i < Dp; i += SA_WAVE) {
-        TA o = zero;
-        if (i < Dv) {
-          float v = to_float(x[i]);
-          if (f) v = (1.f - lambda) * v + lambda * to_float(f[i]);
-          o = from_float<TA>(v);
-        }
-        dst[(size_t)i * page_size] = o;
+// eight consecutive elements from an address that is aligned for them
+__device__ __forceinline__ void load8(const float* p, float (&v)[8]) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+__device__ __forceinline__ void load8(const bf16_t* p, float (&v)[8]) {
+  const uint4 a = *reinterpret_cast<const uint4*>(p);
+  const uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    v[2 * k] = bf16_bits_to_float(w[k] & 0xffffu);
+    v[2 * k + 1] = bf16_bits_to_float(w[k] >> 16);
+  }
+}
+__device__ __forceinline__ void store8(float* p, const float (&v)[8]) {
+  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+}
+__device__ __forceinline__ void store8(bf16_t* p, const float (&v)[8]) {
+  uint32_t w[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k)
+    w[k] = (uint32_t)float_to_bf16_bits(v[2 * k]) | ((uint32_t)float_to_bf16_bits(v[2 * k + 1]) << 16);
+  *reinterpret_cast<uint4*>(p) = make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+// D, Dv, Dp, the row strides multiples of 8, 16-byte aligned bases.  LPH lanes a head (a power of two, 8 LPH >= Dp).
+// Blocks 0 .. qk_blocks - 1: the (token, query or key head) pairs, 256 / LPH a block.  The blocks behind them: the
+// values, a thread per (token, key/value head, 8 dims), tokens fastest.
+template <typename TA, int LPH>
+__global__ __launch_bounds__(256) void qk_norm_kv_write_vec_kernel(
+    const TA* __restrict__ qkv, int row_stride, TA* __restrict__ q_out, const int* __restrict__ positions,
+    const int* __restrict__ slot, TA* __restrict__ k_pages, TA* __restrict__ v_pages, const float* __restrict__ wq,
+    const float* __restrict__ wk, float eps, float temp_coef, int temp_every, const TA* __restrict__ v_first,
+    int v_first_stride, float lambda, int T, int Hq, int Hk, int D, int Dv, int Dp, int page_size, int qk_blocks) {
+  if ((int)blockIdx.x < qk_blocks) {
+    const int sub = threadIdx.x % LPH;
+    const long long unit = (long long)blockIdx.x * (256 / LPH) + threadIdx.x / LPH;
+    const bool live = unit < (long long)T * (Hq + Hk);
+    const long long uc = live ? unit : 0;
+    const int t = (int)(uc / (Hq + Hk)), u = (int)(uc - (long long)t * (Hq + Hk));
+    const bool is_q = u < Hq;
+    const int i = sub * 8;
+    float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (live && i < D) load8(qkv + (size_t)t * row_stride + (size_t)u * D + i, v);
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) ss += v[k] * v[k];
+#pragma unroll
+    for (int o = LPH / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, SA_WAVE);
+    if (!live || i >= Dp) return;
+    const float rs = 1.0f / sqrtf(ss / (float)D + eps);
+    const float temp = is_q ? query_temp(positions, t, temp_coef, temp_every) : 1.f;
+    if (i < D) {
+      float w[8];
+      load8((is_q ? wq : wk) + i, w);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        v[k] = (v[k] * rs) * w[k];
+        if (is_q) v[k] *= temp;
       }
     }
+    if (is_q) {
+      store8(q_out + ((size_t)t * Hq + u) * Dp + i, v);
+    } else {
+      const int s = slot ? slot[t] : -1;
+      if (s < 0) return;
+      const int page = s / page_size, off = s - page * page_size;
+      store8(k_pages + (((size_t)page * Hk + (u - Hq)) * page_size + off) * Dp + i, v);
+    }
+    return;
   }
+  if (!slot) return;
+  const int chunks = Dp >> 3;
+  const long long idx = (long long)(blockIdx.x - qk_blocks) * 256 + threadIdx.x;
+  if (idx >= (long long)T * Hk * chunks) return;
+  const int t = (int)(idx % T);
+  const int gc = (int)(idx / T);
+  const int g = gc / chunks, i = (gc - g * chunks) * 8;
+  const int s = slot[t];
+  if (s < 0) return;
+  const int page = s / page_size, off = s - page * page_size;
+  float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  if (i < Dv) {
+    load8(qkv + (size_t)t * row_stride + (size_t)(Hq + Hk) * D + (size_t)g * Dv + i, v);
+    if (v_first) {
+      float f[8];
+      load8(v_first + (size_t)t * v_first_stride + (size_t)g * Dv + i, f);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) v[k] = (1.f - lambda) * v[k] + lambda * f[k];
+    }
+  }
+  TA* dst = v_pages + (((size_t)page * Hk + g) * Dp + i) * page_size + off;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) dst[(size_t)k * page_size] = from_float<TA>(v[k]);
+}
+
+template <typename TA>
+static int launch_qk_norm(const void* qkv, int row_stride, void* q_out, const int* positions, const int* slot,
+                          void* k_pages, void* v_pages, const float* wq, const float* wk, float eps, float temp_coef,
+                          int temp_every, const void* v_first, int v_first_stride, float lambda, int T, int Hq, int Hk,
+                          int D, int Dv, int Dp, int page_size, hipStream_t stream) {
+  const uintptr_t bits = (uintptr_t)qkv | (uintptr_t)q_out | (uintptr_t)k_pages | (uintptr_t)v_pages |
+                         (uintptr_t)v_first | (uintptr_t)wq | (uintptr_t)wk;
+  const bool vec = ((D | Dv | Dp | row_stride | v_first_stride) & 7) == 0 && (bits & 15) == 0 && Dp <= 512;
+  if (vec) {
+    int lph = 2;
+    while (lph * 8 < Dp) lph *= 2;
+    const long long units = (long long)T * (Hq + Hk), per = 256 / lph;
+    const long long qk_blocks = (units + per - 1) / per;
+    const long long v_blocks = slot ? ((long long)T * Hk * (Dp >> 3) + 255) / 256 : 0;
+    if (qk_blocks + v_blocks > 0x7fffffffLL) return SA_ERR_ARG;
+    dim3 grid((unsigned)(qk_blocks + v_blocks)), block(256);
+#define GOV(LPH)                                                                                                      \
+  hipLaunchKernelGGL((qk_norm_kv_write_vec_kernel<TA, LPH>), grid, block, 0, stream, (const TA*)qkv, row_stride,       \
+                     (TA*)q_out, positions, slot, (TA*)k_pages, (TA*)v_pages, wq, wk, eps, temp_coef, temp_every,     \
+                     (const TA*)v_first, v_first_stride, lambda, T, Hq, Hk, D, Dv, Dp, page_size, (int)qk_blocks)
+    switch (lph) {
+      case 2: GOV(2); break;
+      case 4: GOV(4); break;
+      case 8: GOV(8); break;
+      case 16: GOV(16); break;
+      case 32: GOV(32); break;
+      default: GOV(64); break;
+    }
+#undef GOV
+    return 0;
+  }
+  const int units = Hq + 2 * Hk;
+  if ((units + 3) / 4 > 65535) return SA_ERR_ARG;
+  dim3 grid(T, (units + 3) / 4), block(256);
+  hipLaunchKernelGGL(qk_norm_kv_write_kernel<TA>, grid, block, 0, stream, (const TA*)qkv, row_stride, (TA*)q_out,
+                     positions, slot, (TA*)k_pages, (TA*)v_pages, wq, wk, eps, temp_coef, temp_every,
+                     (const TA*)v_first, v_first_stride, lambda, Hq, Hk, D, Dv, Dp, page_size);
+  return 0;
 }
 
 extern "C" int sa_qk_norm_kv_write(const void* qkv, int row_stride, void* q_out, int act_dtype, const int* positions,
@@ -88,15 +229,16 @@ extern "C" int sa_qk_norm_kv_write(const void* qkv, int row_stride, void* q_out,
     return SA_ERR_ARG;
   if (row_stride < Hq * D + Hk * (D + Dv) || (slot && (!k_pages || !v_pages)) || (temp_every > 0 && !positions))
     return SA_ERR_ARG;
-  dim3 grid(T), block(256);
-#define GO(TA)                                                                                                        \
-  hipLaunchKernelGGL(qk_norm_kv_write_kernel<TA>, grid, block, 0, stream, (const TA*)qkv, row_stride, (TA*)q_out,     \
-                     positions, slot, (TA*)k_pages, (TA*)v_pages, wq, wk, eps, temp_coef, temp_every,                 \
-                     (const TA*)v_first, v_first_stride, lambda, Hq, Hk, D, Dv, Dp, page_size)
-  if (act_dtype == SA_F32) GO(float);
-  else if (act_dtype == SA_BF16) GO(bf16_t);
-  else return SA_ERR_UNSUPPORTED;
-#undef GO
+  int rc;
+  if (act_dtype == SA_F32)
+    rc = launch_qk_norm<float>(qkv, row_stride, q_out, positions, slot, k_pages, v_pages, wq, wk, eps, temp_coef,
+                               temp_every, v_first, v_first_stride, lambda, T, Hq, Hk, D, Dv, Dp, page_size, stream);
+  else if (act_dtype == SA_BF16)
+    rc = launch_qk_norm<bf16_t>(qkv, row_stride, q_out, positions, slot, k_pages, v_pages, wq, wk, eps, temp_coef,
+                                temp_every, v_first, v_first_stride, lambda, T, Hq, Hk, D, Dv, Dp, page_size, stream);
+  else
+    return SA_ERR_UNSUPPORTED;
+  if (rc != 0) return rc;
   SA_LAUNCH_CHECK();
   return 0;
 }

@@ -265,15 +265,17 @@ def test_greedy_generation_through_the_scheduler(tmp_path, name, dtype):
 # the kernels alone
 # ---------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,G,D,Dv,Dp", [(4, 2, 16, 16, 16), (6, 1, 24, 40, 48), (3, 3, 10, 7, 16), (2, 1, 136, 20, 144)])
-def test_qk_norm_kv_write(dtype, H, G, D, Dv, Dp):
+@pytest.mark.parametrize("pad", [5, 8])      # rows that do not keep 16-byte alignment (the general kernel), and rows that do
+@pytest.mark.parametrize("H,G,D,Dv,Dp", [(4, 2, 16, 16, 16), (6, 1, 24, 40, 48), (3, 3, 10, 7, 16), (2, 1, 136, 24, 144),
+                                         (5, 5, 128, 64, 128)])
+def test_qk_norm_kv_write(dtype, H, G, D, Dv, Dp, pad):
     from serve_amd import ops
     torch.manual_seed(D)
     T, page, P = 11, 4, 9
     width = H * D + G * (D + Dv)
-    wide = torch.randn(T, width + 5, device="cuda").to(dtype)               # rows inside wider rows
+    wide = torch.randn(T, width + pad, device="cuda").to(dtype)             # rows inside wider rows
     qkv = wide[:, :width]
-    first = torch.randn(T, G * Dv + 3, device="cuda").to(dtype)[:, : G * Dv]
+    first = torch.randn(T, G * Dv + pad, device="cuda").to(dtype)[:, : G * Dv]
     wq, wk = torch.rand(D, device="cuda") + 0.5, torch.rand(D, device="cuda") + 0.5
     positions = torch.tensor([0, 1, 2, 3, 4, 5, 6, 7, 30, 31, 32], dtype=torch.int32, device="cuda")
     slots = torch.tensor([5, 6, 7, 8, 20, 21, 22, 23, -1, 1, 35], dtype=torch.int32, device="cuda")

@@ -156,3 +156,23 @@ def test_plain_model_is_causal_and_mechanisms_show(tmp_path):
     d = moved(config=late)
     # (one position in five has another temperature in one layer of four: the float32 comparison is the one that tells)
     assert d[:4].max() == 0.0 and (d[4:] > 20 * tm.TOLERANCE["float32"]).float().mean() > 0.8
+
+
+def test_random_model_from_the_command_line(tmp_path):
+    """`random-model` writes a folder for the named shape, and again from that folder's config.json: the same
+    tensors (a pure function of seed and tensor name), which the plain model can run."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    a, b = str(tmp_path / "a"), str(tmp_path / "b")
+    run = lambda *args: subprocess.run([sys.executable, "-m", "serve_amd", "random-model", *args], cwd=root,   # noqa: E731
+                                       capture_output=True, text=True, timeout=300)
+    p = run("--shape", "timopel-tiny", "--out", a, "--seed", "5")
+    assert p.returncode == 0, p.stderr[-2000:]
+    p = run("--config", os.path.join(a, "config.json"), "--out", b, "--seed", "5")
+    assert p.returncode == 0, p.stderr[-2000:]
+    wa, wb = tm.plain_weights(a), tm.plain_weights(b)
+    assert sorted(wa) == sorted(wb) and all(torch.equal(wa[k], wb[k]) for k in wa)
+    logits = tp.forward([1, 2, 3, 4, 5], wa, tm.plain_config(a))
+    assert logits.shape == (5, 512) and torch.isfinite(logits).all()

@@ -18,7 +18,7 @@ from tests.plain import timopel_plain as tp
 pytestmark = pytest.mark.gpu
 
 DTYPES = ["float32", "bfloat16"]
-NAMES = ["TA", "TB", "TC", "TD"]
+NAMES = ["TA", "TB", "TC", "TD", "TE"]
 
 
 def tokens_for(n, seed, vocab):
@@ -510,3 +510,17 @@ def test_traces_through_the_program(tmp_path, dtype):
     assert sum(len(t) for t in reqs.values()) > 256          # pages went from request to request
     for k, t in reqs.items():
         tm.assert_matches_plain(torch.cat(rows[k]), folder, t, dtype, f"trace request {k}")
+
+
+def test_generate_from_the_command_line():
+    """`python -m serve_amd generate` with the named shape: as many token lists as prompts, of the asked length."""
+    import json
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([sys.executable, "-m", "serve_amd", "generate", "--shape", "timopel-tiny", "--random-prompts", "3:20",
+                           "--max-new-tokens", "6", "--temperature", "0"], cwd=root, capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    lines = [json.loads(l) for l in proc.stdout.splitlines() if l.startswith("[")]
+    assert len(lines) == 3 and all(len(l) == 6 and all(0 <= t < 512 for t in l) for l in lines)

@@ -11,6 +11,8 @@ The models differ in every size and option:
       101, experts of width 9 of which all are taken (top = experts = 3), nobody blends
   TD  keys of 136 (a cache head of 144: above what the matrix-core and tiled attention kernels take), values of
       20, 2 heads on one key/value head
+  TE  20 heads on one key/value head (more rows a key/value head than the kernels for single tokens take), a layer
+      that does not blend between two that do, top 2 of 9 experts without a shared one
 """
 from __future__ import annotations
 
@@ -55,7 +57,13 @@ TD = TimopelConfig(vocab=120, width=64, eps=1e-5, residual_mult=0.3, embedding_s
     L(_att(2, 1, 136, 20, 0.15, (0.3, 16), v_mix=True), None),
 ))
 
-MODELS = {"TA": (TA, 3), "TB": (TB, 4), "TC": (TC, 5), "TD": (TD, 6)}
+TE = TimopelConfig(vocab=130, width=80, eps=1e-5, residual_mult=0.5, embedding_scale=1.5, layers=(
+    L(_att(20, 1, 32, 32, 0.2, (0.3, 4), v_mix=True), ClampedMoeConfig(9, 2, 2.0, 16, 1.2)),
+    L(_att(20, 1, 32, 32, 0.2, (0.3, 4), v_mix=False), GatedDenseConfig(48)),
+    L(_att(20, 1, 32, 32, 0.2, (0.3, 4), v_mix=True), None),
+))
+
+MODELS = {"TA": (TA, 3), "TB": (TB, 4), "TC": (TC, 5), "TD": (TD, 6), "TE": (TE, 7)}
 
 # the embedding at a scale at which the logits (the table is the output matrix too) are of order one, and sinks
 # that weigh as much as dozens of keys in some heads

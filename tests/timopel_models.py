@@ -12,7 +12,7 @@ The models differ in every size and option:
   TD  keys of 136 (a cache head of 144: above what the matrix-core and tiled attention kernels take), values of
       20, 2 heads on one key/value head
   TE  20 heads on one key/value head (more rows a key/value head than the kernels for single tokens take), a layer
-      that does not blend between two that do, top 2 of 9 experts without a shared one
+      that does not blend between two that do, top 2 of 9 experts
 """
 from __future__ import annotations
 
@@ -57,8 +57,8 @@ TD = TimopelConfig(vocab=120, width=64, eps=1e-5, residual_mult=0.3, embedding_s
     L(_att(2, 1, 136, 20, 0.15, (0.3, 16), v_mix=True), None),
 ))
 
-TE = TimopelConfig(vocab=130, width=80, eps=1e-5, residual_mult=0.5, embedding_scale=1.5, layers=(
-    L(_att(20, 1, 32, 32, 0.2, (0.3, 4), v_mix=True), ClampedMoeConfig(9, 2, 2.0, 16, 1.2)),
+TE = TimopelConfig(vocab=130, width=80, eps=1e-5, residual_mult=0.3, embedding_scale=1.5, layers=(
+    L(_att(20, 1, 32, 32, 0.2, (0.3, 4), v_mix=True), ClampedMoeConfig(9, 2, 1.0, 16, 1.2, 24, 1.2)),
     L(_att(20, 1, 32, 32, 0.2, (0.3, 4), v_mix=False), GatedDenseConfig(48)),
     L(_att(20, 1, 32, 32, 0.2, (0.3, 4), v_mix=True), None),
 ))

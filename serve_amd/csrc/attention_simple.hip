@@ -6,7 +6,8 @@
 // scores = q.k * scale, key j visible to the query at absolute position p iff j <= p (and
 // p - j < window when a window is set), online softmax (m, l, O), O / l at the end.  Query head
 // h reads KV head h / (Hq / Hk).  With `sinks` (fp32 [Hq], or null) the softmax of head h has one more
-// term exp(sinks[h]) in its denominator, which has no key and no value and is not scaled: it joins l
+// term exp(sinks[h]) in its denominator (sinks[h] as it is stored: `scale` does not apply to it), which takes
+// weight away from the keys and adds nothing to the output: it joins l
 // when a row is finished (once per row: in the merge where the key range was cut).
 //
 // Batch layout: the T tokens of a step are the concatenation of B segments; segment r covers

@@ -235,8 +235,8 @@ SIMPLE_ATTENTION_MAX_HEAD_DIM = 640     # (SA_MAX_D of csrc/attention_simple.hip
 
 
 def _check_sinks(sinks: Optional[torch.Tensor], num_heads: int) -> None:
-    """`sinks`: per query head one more term exp(sinks[h]) in the softmax's denominator, with no key and
-    no value (fp32 [Hq] on the device); None: a plain softmax."""
+    """`sinks`: per query head one more term exp(sinks[h]) in the softmax's denominator, which takes weight
+    away from the keys and adds nothing to the output (fp32 [Hq] on the device); None: a plain softmax."""
     if sinks is not None:
         _check(sinks.is_cuda and sinks.is_contiguous() and sinks.dtype == torch.float32
                and sinks.numel() == num_heads, f"sinks must be contiguous fp32 [{num_heads}] on the GPU")

@@ -85,23 +85,15 @@ __device__ __forceinline__ void route_token(const float* __restrict__ z, int* __
 // ---------------------------------------------------------------------------------------------
 // group: one workgroup.  Counts per expert, their running sum, the tiles, then every (token, k)
 // takes the next free row of its expert (the order inside an expert does not matter: a row's sums
-// do not depend on its place).
+// do not depend on its place).  Up to MOE_LDS_EXPERTS experts the counters live in LDS, whose atomics
+// on a few dozen addresses are far cheaper than the same through memory (thousands of rows of a prompt
+// step on 32 experts: 64 us with the counters in memory).
 // ---------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(1024) void moe_group_kernel(const int* ids, int n, int E, int tile_rows,
-                                                         int* __restrict__ offsets, int* __restrict__ cursor,
-                                                         int* __restrict__ perm, int* __restrict__ tile_expert,
-                                                         int* __restrict__ tile_row0, int* __restrict__ num_tiles,
-                                                         const float* __restrict__ logits, int ldz, int* ids_out,
-                                                         float* __restrict__ wts, int top, int over_all, float wscale) {
-  for (int e = threadIdx.x; e < E; e += blockDim.x) cursor[e] = 0;
-  if (logits) {
-    // a step of few tokens: the routing is done here, a wave a token in turn, and saves a kernel
-    const int waves = blockDim.x / SA_WAVE, T = n / top;
-    for (int t = threadIdx.x / SA_WAVE; t < T; t += waves)
-      route_token(logits + (size_t)t * ldz, ids_out + (size_t)t * top, wts + (size_t)t * top, E, top,
-                  threadIdx.x & (SA_WAVE - 1), over_all, wscale);
-  }
-  __syncthreads();
+#define MOE_LDS_EXPERTS 1024
+// counts, running sums and tiles, then the rows' places; `cursor`: E counters, in LDS or in memory
+__device__ __forceinline__ void group_rows(const int* ids, int n, int E, int tile_rows, int* __restrict__ offsets,
+                                           int* cursor, int* __restrict__ perm, int* __restrict__ tile_expert,
+                                           int* __restrict__ tile_row0, int* __restrict__ num_tiles) {
   for (int i = threadIdx.x; i < n; i += blockDim.x) atomicAdd(&cursor[ids[i]], 1);
   __syncthreads();
   if (threadIdx.x == 0) {
@@ -122,6 +114,30 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int* ids, int n, 
   }
   __syncthreads();
   for (int i = threadIdx.x; i < n; i += blockDim.x) perm[atomicAdd(&cursor[ids[i]], 1)] = i;
+}
+
+__global__ __launch_bounds__(1024) void moe_group_kernel(const int* ids, int n, int E, int tile_rows,
+                                                         int* __restrict__ offsets, int* __restrict__ cursor,
+                                                         int* __restrict__ perm, int* __restrict__ tile_expert,
+                                                         int* __restrict__ tile_row0, int* __restrict__ num_tiles,
+                                                         const float* __restrict__ logits, int ldz, int* ids_out,
+                                                         float* __restrict__ wts, int top, int over_all, float wscale) {
+  __shared__ int lds_cursor[MOE_LDS_EXPERTS];
+  const bool in_lds = E <= MOE_LDS_EXPERTS;              // (the counters are scratch: nobody reads them afterwards)
+  for (int e = threadIdx.x; e < E; e += blockDim.x) {
+    if (in_lds) lds_cursor[e] = 0;
+    else cursor[e] = 0;
+  }
+  if (logits) {
+    // a step of few tokens: the routing is done here, a wave a token in turn, and saves a kernel
+    const int waves = blockDim.x / SA_WAVE, T = n / top;
+    for (int t = threadIdx.x / SA_WAVE; t < T; t += waves)
+      route_token(logits + (size_t)t * ldz, ids_out + (size_t)t * top, wts + (size_t)t * top, E, top,
+                  threadIdx.x & (SA_WAVE - 1), over_all, wscale);
+  }
+  __syncthreads();
+  if (in_lds) group_rows(ids, n, E, tile_rows, offsets, lds_cursor, perm, tile_expert, tile_row0, num_tiles);
+  else group_rows(ids, n, E, tile_rows, offsets, cursor, perm, tile_expert, tile_row0, num_tiles);
 }
 
 // ---------------------------------------------------------------------------------------------

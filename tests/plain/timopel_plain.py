@@ -110,15 +110,23 @@ def route(z: Tensor, top: int, scale: float) -> (Tensor, Tensor):
     return order, chosen / (chosen.sum(-1, keepdim=True) + 1e-20) * scale
 
 
-def moe_ff(h: Tensor, W: Dict[str, Tensor], mlp: dict) -> Tensor:
+def moe_ff(h: Tensor, W: Dict[str, Tensor], mlp: dict, margins: Optional[list] = None) -> Tensor:
+    """`margins` (a list) receives per token (position, lead of the last chosen logit over the first that is
+    left out, as a share of the logits' spread): how clear the router's choice is."""
     r = mlp["router"]
-    ids, wts = route(h @ W["router"].T, int(r["top"]), float(r["scale"]))
+    z = h @ W["router"].T
+    ids, wts = route(z, int(r["top"]), float(r["scale"]))
+    if margins is not None and int(r["top"]) < z.shape[1]:
+        v = torch.sort(z, dim=-1, descending=True).values
+        lead = (v[:, int(r["top"]) - 1] - v[:, int(r["top"])]) / (v[:, 0] - v[:, -1]).clamp_min(1e-30)
+        margins.extend((t, float(m)) for t, m in enumerate(lead))
     out = torch.zeros_like(h)
     limit = float(mlp["expert"]["limit"])
-    for t in range(h.shape[0]):
-        for j in range(ids.shape[1]):
-            e = int(ids[t, j])
-            out[t] += wts[t, j] * expert_ff(h[t: t + 1], W, f"e{e}.", limit)[0]
+    for e in range(z.shape[1]):
+        took = ids == e                                   # [T, top]: which tokens chose expert e, and at which place
+        rows = took.any(-1)
+        if rows.any():
+            out[rows] += (wts * took).sum(-1, keepdim=True)[rows] * expert_ff(h[rows], W, f"e{e}.", limit)
     if mlp.get("shared"):
         out = out + expert_ff(h, W, "shared.", float(mlp["shared"]["limit"]))
     return out
@@ -132,8 +140,8 @@ def _sub(W: Dict[str, Tensor], prefix: str) -> Dict[str, Tensor]:
 
 
 def forward(tokens: Sequence[int], weights: Dict[str, Tensor], cfg: dict, dtype=torch.float64,
-            return_layers: bool = False):
-    """Logits [T, vocab] of one sequence from position 0 (and the stream after every layer)."""
+            return_layers: bool = False, margins: Optional[list] = None):
+    """Logits [T, vocab] of one sequence from position 0 (and the stream after every layer).  `margins`: see moe_ff."""
     W = {k: v.to(dtype) for k, v in weights.items()}
     eps = float(cfg["norm"]["eps"])
     c = float(cfg["residual_mult"])
@@ -158,7 +166,7 @@ def forward(tokens: Sequence[int], weights: Dict[str, Tensor], cfg: dict, dtype=
             if mlp["kind"] == "dense":
                 y = dense_ff(h, M)
             elif mlp["kind"] == "moe":
-                y = moe_ff(h, M, mlp)
+                y = moe_ff(h, M, mlp, margins)
             else:
                 raise ValueError(f"layer {i}: unknown feed-forward {mlp['kind']!r}")
             x = x + c * rms_norm(y, L["norm2b"], eps)

@@ -62,9 +62,10 @@ def test_tensor_names_and_shapes():
     model = Model(build_timopel_spec(tm.TA))
     req = {r.checkpoint_name: tuple(r.shape) for r in model.weight_requests() if not r.alias_only}
     assert req["embed"] == (150, 64) and req["final.norm"] == (64,)
-    assert req["l0.mix.q"] == (64, 64) and req["l0.mix.k"] == (32, 64) and req["l0.mix.v"] == (32, 64)
-    assert req["l0.mix.q.norm"] == (16,) and req["l0.mix.k.norm"] == (16,) and req["l0.mix.sink"] == (4,)
-    assert req["l0.mix.o"] == (64, 64)
+    assert req["l0.mix.q"] == (64, 64) and req["l0.mix.k"] == (32, 64) and req["l0.mix.v"] == (8, 64)
+    assert req["l0.mix.q.norm"] == (32,) and req["l0.mix.k.norm"] == (32,) and req["l0.mix.sink"] == (2,)
+    assert req["l0.mix.o"] == (64, 16)
+    assert req["l1.mix.q"] == (64, 64) and req["l1.mix.v"] == (32, 64) and req["l1.mix.sink"] == (4,) and req["l1.mix.o"] == (64, 64)
     assert "l0.mix.vmix" not in req and req["l1.mix.vmix"] == () and req["l3.mix.vmix"] == ()
     assert req["l0.mlp.gate"] == (96, 64) and req["l0.mlp.down"] == (64, 96)
     assert req["l1.mlp.router"] == (6, 64) and req["l1.mlp.e5.up"] == (24, 64) and req["l1.mlp.shared.down"] == (64, 40)
@@ -83,9 +84,11 @@ def test_who_blends_with_whom_and_what_is_cached():
     assert [l.ffn is None for l in model.layers] == [False, False, True, False]
     assert model.graph_safe()
     # keys of 24 and values of 40 share cache heads of 48; keys of 136 heads of 144
-    for cfg, size, kv in ((tm.TB, 48, 1), (tm.TD, 144, 1), (tm.TC, 16, 3), (tm.TA, 16, 2)):
+    for cfg, size, kv in ((tm.TB, 48, 1), (tm.TD, 144, 1), (tm.TC, 16, 3)):
         reqs = Model(build_timopel_spec(cfg)).cache_requests()
         assert all(r.window is None and [t.shape for t in r.tensors] == [(kv, size), (kv, size)] for r in reqs)
+    reqs = Model(build_timopel_spec(tm.TA)).cache_requests()         # layers with cache heads of different sizes
+    assert [[t.shape for t in r.tensors] for r in reqs] == [[(1, 32), (1, 32)]] + [[(2, 16), (2, 16)]] * 3
     assert all(s is None for s in model.state_requests())
 
 

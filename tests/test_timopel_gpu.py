@@ -21,7 +21,11 @@ DTYPES = ["float32", "bfloat16"]
 NAMES = ["TA", "TB", "TC", "TD", "TE"]
 
 
-def tokens_for(n, seed, vocab):
+def tokens_for(n, seed, vocab, folder=None, dtype="float32"):
+    """Random tokens; for a comparison in bfloat16 of a model with routers (`folder` given), tokens whose routing
+    decisions are all clear in the plain model, so that the comparison does not rest on a close call."""
+    if folder is not None and dtype == "bfloat16":
+        return tm.clear_tokens(folder, n, seed, vocab)
     rng = random.Random(seed)
     return [rng.randrange(vocab) for _ in range(n)]
 
@@ -33,7 +37,7 @@ def test_whole_prompts_and_first_tokens(tmp_path, name, dtype):
     engine = tm.engine_for(folder, dtype)
     vocab = tm.MODELS[name][0].vocab
     for n in (1, 2, 3, 5, 61):
-        tokens = tokens_for(n, 100 + n, vocab)
+        tokens = tokens_for(n, 100 + n, vocab, folder, dtype)
         got = tm.run_portions(engine, f"r{n}", tokens, [n])
         tm.assert_matches_plain(got, folder, tokens, dtype, f"{name} whole {n}")
     engine.runner.cache.check_invariants()
@@ -45,7 +49,7 @@ def test_prompt_then_token_by_token(tmp_path, name, dtype):
     folder = tm.make_folder(tmp_path, name)
     engine = tm.engine_for(folder, dtype)
     vocab = tm.MODELS[name][0].vocab
-    tokens = tokens_for(84, 7, vocab)
+    tokens = tokens_for(84, 7, vocab, folder, dtype)
     got = tm.run_portions(engine, "r", tokens, [84 - 45] + [1] * 45)     # temperature steps pass under decoded tokens
     tm.assert_matches_plain(got, folder, tokens, dtype, f"{name} prompt + 45 single tokens")
     got = tm.run_portions(engine, "s", tokens[:30], [1] * 30)             # from the very first token on
@@ -61,7 +65,7 @@ def test_portions_of_changing_size(tmp_path, name, dtype):
     folder = tm.make_folder(tmp_path, name)
     engine = tm.engine_for(folder, dtype)
     vocab = tm.MODELS[name][0].vocab
-    tokens = tokens_for(73, 8, vocab)
+    tokens = tokens_for(73, 8, vocab, folder, dtype)
     for portions in ([7, 2, 16, 3, 2, 9, 2, 11, 5, 4, 1, 1, 2, 8], [2] * 10 + [53], [1, 3, 69], [40, 33]):
         got = tm.run_portions(engine, "r", tokens, portions)
         tm.assert_matches_plain(got, folder, tokens, dtype, f"{name} portions {portions}")
@@ -99,7 +103,7 @@ def test_unequal_requests_together_with_pages_and_slots_used_again(tmp_path, nam
     # four live requests of at most 41 tokens: pool and slots are far fewer than the requests need together
     engine = tm.engine_for(folder, dtype, num_pages=4 * 11 + 1, page_size=4, max_requests=4)
     vocab = tm.MODELS[name][0].vocab
-    reqs = {f"q{i}": tokens_for(n, 300 + i, vocab) for i, n in enumerate(lengths)}
+    reqs = {f"q{i}": tokens_for(n, 300 + i, vocab, folder, dtype) for i, n in enumerate(lengths)}
     steps = mixed_trace(random.Random(13), reqs)
     rows = {k: [] for k in reqs}
     slots_seen, pages_seen = {}, {}
@@ -220,7 +224,7 @@ def test_long_decoding(tmp_path, name, dtype):
     folder = tm.make_folder(tmp_path, name)
     engine = tm.engine_for(folder, dtype, num_pages=80)
     vocab = tm.MODELS[name][0].vocab
-    tokens = tokens_for(260, 31, vocab)
+    tokens = tokens_for(260, 31, vocab, folder, dtype)
     got = tm.run_portions(engine, "r", tokens, [4] + [1] * 256)
     tm.assert_matches_plain(got, folder, tokens, dtype, f"{name} 256 single tokens")
 
@@ -234,7 +238,7 @@ def test_greedy_generation_through_the_scheduler(tmp_path, name, dtype):
     folder = tm.make_folder(tmp_path, name)
     engine = tm.engine_for(folder, dtype, num_pages=128, page_size=8, max_requests=3)
     vocab = tm.MODELS[name][0].vocab
-    prompts = [tokens_for(n, 50 + n, vocab) for n in (5, 19, 1, 33, 8)]
+    prompts = [tokens_for(n, 50 + n, vocab, folder, dtype) for n in (5, 19, 1, 33, 8)]
     new = 12
     reqs = [Request(torch.tensor(p), len(p), new) for p in prompts]
     out = engine.generate(reqs, temperature=0.0, return_logits="all")
@@ -481,7 +485,7 @@ def test_traces_through_the_program(tmp_path, dtype):
     reqs, steps = {}, []
 
     def feed(key, n, portions, seed):
-        reqs[key] = tokens_for(n, seed, vocab)
+        reqs[key] = tokens_for(n, seed, vocab, folder, dtype)
         at = 0
         for j, m in enumerate(portions):
             steps.append(([(key, reqs[key][at: at + m])], [key] if j == len(portions) - 1 else []))
@@ -490,7 +494,7 @@ def test_traces_through_the_program(tmp_path, dtype):
     feed("whole", 50, [50], 1)
     feed("tail", 70, [30] + [1] * 40, 2)
     feed("cut", 61, [7, 2, 16, 3, 2, 9, 2, 11, 5, 4], 3)
-    mixed = {f"m{i}": tokens_for(n, 40 + i, vocab) for i, n in enumerate([23, 41, 9, 30, 17, 2, 36, 12, 40])}
+    mixed = {f"m{i}": tokens_for(n, 40 + i, vocab, folder, dtype) for i, n in enumerate([23, 41, 9, 30, 17, 2, 36, 12, 40])}
     reqs.update(mixed)
     steps.extend(mixed_trace(random.Random(5), mixed))
     lines = [json.dumps({"step": i, "entries": [{"id": k, "tokens": t, "want": list(range(len(t)))} for k, t in entries],

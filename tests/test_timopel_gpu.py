@@ -528,3 +528,46 @@ def test_generate_from_the_command_line():
     assert proc.returncode == 0, proc.stderr[-3000:]
     lines = [json.loads(l) for l in proc.stdout.splitlines() if l.startswith("[")]
     assert len(lines) == 3 and all(len(l) == 6 and all(0 <= t < 512 for t in l) for l in lines)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_steps_with_prompt_portions_replayed_from_graphs(tmp_path, dtype):
+    """Six slots and portions of eight tokens: steps of a few decoding requests in front of prompt portions come
+    again and again, are padded with inert segments (no pages, no slot: nothing of them is stored) and replayed from
+    graphs; the greedy tokens are those of the same schedule launched kernel by kernel, and the plain model's where
+    its choice is clear."""
+    from serve_amd.engine.engine import Request
+    name = "TA"
+    folder = tm.make_folder(tmp_path, name)
+    vocab = tm.MODELS[name][0].vocab
+    rng = random.Random(46)
+    count = 30
+    prompts = [tokens_for(rng.randrange(9, 30), 700 + i, vocab, folder, dtype) for i in range(count)]
+    new = [rng.randrange(4, 12) for _ in range(count)]
+    kw = dict(num_pages=64, page_size=8, max_requests=6)
+    outs = []
+    for mixed in (True, False):
+        from serve_amd.config.engine import EngineConfig
+        from serve_amd.engine.engine import Engine
+        engine = Engine.from_folder(folder, EngineConfig(dtype=dtype, max_context=256, max_tokens_per_step=24, prefill_chunk=8,
+                                                         graph_mixed_steps=mixed, **kw))
+        out = engine.generate([Request(torch.tensor(p), len(p), n) for p, n in zip(prompts, new)], temperature=0.0)
+        assert all(r.error is None and len(r.generated_tokens) == n for r, n in zip(out, new))
+        graphs = [k for k, e in engine.runner._graphs.items() if k[0] == "mixed" and e.graph is not None and e.launches > 2]
+        assert bool(graphs) == mixed, f"mixed graphs {mixed}: replayed shapes {graphs}"
+        engine.runner.cache.check_invariants()
+        outs.append([r.generated_tokens.tolist() for r in out])
+    if dtype == "float32":
+        assert outs[0] == outs[1]
+    compared = 0
+    for p, got in zip(prompts, outs[0]):
+        seq = list(p)
+        for tok in got:
+            row = tm.plain_logits(folder, seq)[-1]
+            top2 = row.topk(2).values
+            if (top2[0] - top2[1]).item() < (1e-3 if dtype == "float32" else 0.15):
+                break
+            assert tok == int(row.argmax())
+            seq.append(tok)
+            compared += 1
+    assert compared > 3 * count

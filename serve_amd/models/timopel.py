@@ -69,6 +69,9 @@ def build_timopel_spec(cfg: TimopelConfig) -> ModelSpec:
         lm_head=PartSpec("linear_head", {"vocab_size": cfg.vocab, "hidden_size": d, "tied": True,
                                          "shares": "embedding.weight"}),
         weights={"embedding.weight": "embed", "final_norm.weight": "final.norm", "lm_head.weight": "embed"},
+        # a checkpoint may carry the blending scalar of a layer that does not blend, and the feed-forward's norms of
+        # a layer without feed-forward: nothing reads them
+        ignored_weight_patterns=[r"l\d+\.mix\.vmix", r"l\d+\.norm2b?"],
     )
 
 

@@ -60,7 +60,8 @@ class QKNormAttention(Part):
                ParamRequest("v", (G * Dv, d), init="normal:0.08"),
                ParamRequest("q.norm", (D,), init="ones_normal:0.2"), ParamRequest("k.norm", (D,), init="ones_normal:0.2")]
         if self.v_blend != "none":
-            out.append(ParamRequest("vmix", (), init="uniform:0.2:0.6"))     # (read by the blending layers only)
+            # (read by the blending layers only: the source layer's may be missing)
+            out.append(ParamRequest("vmix", (), init="uniform:0.2:0.6", optional=self.v_blend == "source"))
         if self.sink:
             out.append(ParamRequest("sink", (H,), init="normal:1.0"))
         return out + [ParamRequest("o", (d, H * Dv), init="normal:0.08")]

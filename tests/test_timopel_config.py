@@ -179,3 +179,21 @@ def test_random_model_from_the_command_line(tmp_path):
     assert sorted(wa) == sorted(wb) and all(torch.equal(wa[k], wb[k]) for k in wa)
     logits = tp.forward([1, 2, 3, 4, 5], wa, tm.plain_config(a))
     assert logits.shape == (5, 512) and torch.isfinite(logits).all()
+
+
+def test_checkpoint_tensors_that_nothing_reads_are_tolerated():
+    """A blending scalar in a layer that does not blend and second-half norms in a layer without feed-forward are
+    ignored; the first blending layer's scalar may be missing; anything else that is unexpected or missing is an error."""
+    from serve_amd.weights.loader import WeightError, check_against, random_reader
+    model = Model(build_timopel_spec(tm.TA))
+    reader = random_reader(model, 1)
+    reader._t["l0.mix.vmix"] = torch.tensor(0.5)
+    reader._t["l2.norm2"] = torch.ones(64)
+    reader._t["l2.norm2b"] = torch.ones(64)
+    del reader._t["l1.mix.vmix"]
+    check_against(model, reader)
+    reader._t["l2.mlp.gate"] = torch.ones(4, 64)
+    del reader._t["l3.mix.vmix"]
+    with pytest.raises(WeightError) as e:
+        check_against(model, reader)
+    assert e.value.unexpected == ["l2.mlp.gate"] and e.value.missing == ["l3.mix.vmix"]

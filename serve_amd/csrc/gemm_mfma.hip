@@ -52,6 +52,21 @@ struct QkvRopeArgs {
   float gate_limit;
 };
 
+// Routed experts through gemm_wide_kernel: the rows of a workgroup are a tile of one expert's rows, from lists
+// that a kernel of csrc/moe.hip has built on the device (offsets[E + 1]: first grouped row of every expert;
+// perm: grouped row -> token * top + k; tile_expert, tile_row0, num_tiles).  MOE 1: activations are gathered
+// (row perm[r] / top of A), weights are expert e's N rows of W ([2, E, N, K]: gates, then ups), the gated sums go
+// to row r of C.  MOE 2: activations are the grouped rows themselves, weights expert e's N rows of W [E, N, K],
+// the sums go to row perm[r] of C.
+struct MoeTileArgs {
+  const int* offsets;
+  const int* perm;
+  const int* tile_expert;
+  const int* tile_row0;
+  const int* num_tiles;
+  int top;
+};
+
 // silu(g) u with the fast exponential, as the plain SwiGLU feed-forward has always been computed; any other gate
 // through gate_mul
 __device__ __forceinline__ float gated(float gt, float up, const QkvRopeArgs& qa) {
@@ -545,10 +560,10 @@ static int launch_mid(const void* A, const void* W, void* C, int M, int N, int K
 // read from the last row and their sums never stored.
 #define SA_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xf) | (((n) >> 4) << 14) | (0x7 << 4) | (0xf << 8))
 
-template <int MW, int NT, int NB, typename TC, int EPI, int SPB = 1>
+template <int MW, int NT, int NB, typename TC, int EPI, int SPB = 1, int MOE = 0>
 __global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
                                                        TC* __restrict__ C, int M, int N, int K, int up_offset,
-                                                       QkvRopeArgs qa) {
+                                                       QkvRopeArgs qa, MoeTileArgs ma) {
   constexpr bool SWIGLU = EPI == EPI_SWIGLU;
   constexpr bool QKV = EPI == EPI_QKV_ROPE;
   static_assert(NT == 1 || NT == 2 || NT == 4 || NT == 8 || NT == 16, "tiles of 16 weight rows, 8 rows a wave and instruction");
@@ -573,8 +588,18 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16_t* __restrict
   const int c = lane & 15;
   const int mw = wave & 3;
   const int kh = wave >> 2;
-  const int m0 = blockIdx.z * BM;
+  const int m0 = MOE ? 0 : blockIdx.z * BM;
   const int n0 = blockIdx.x * COLS;
+  // experts: this workgroup's tile of grouped rows (surplus workgroups of the worst-case grid leave at once)
+  int moe_row0 = 0;
+  if constexpr (MOE != 0) {
+    const int tile = blockIdx.z;
+    if (tile >= *ma.num_tiles) return;
+    const int e = ma.tile_expert[tile];
+    moe_row0 = ma.tile_row0[tile];
+    M = min(BM, ma.offsets[e + 1] - moe_row0);            // rows of this tile
+    W += (size_t)e * N * K;
+  }
   const bool has_w = NT >= 4 || wave < 2 * NT;     // (wave-uniform) whether this wave fetches weight rows
   // the rotating epilogue: a tile holds eight dims of a head and their partners half a head further on
   const int tph = QKV ? (qa.D >> 4) : 1;
@@ -599,7 +624,9 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16_t* __restrict
   for (int d = 0; d < MW; ++d) {
     const int row = (wave * MW + d) * 8 + (lane >> 3);
     const int seg = (lane & 7) ^ ((row >> 1) & 7);
-    src[d] = A + (size_t)min(m0 + row, M - 1) * K + seg * 8;
+    if constexpr (MOE == 1) src[d] = A + (size_t)(ma.perm[moe_row0 + min(row, M - 1)] / ma.top) * K + seg * 8;
+    else if constexpr (MOE == 2) src[d] = A + (size_t)(moe_row0 + min(row, M - 1)) * K + seg * 8;
+    else src[d] = A + (size_t)min(m0 + row, M - 1) * K + seg * 8;
   }
 #pragma unroll
   for (int d = 0; d < NWI; ++d) {
@@ -734,8 +761,10 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16_t* __restrict
   // lane l holds C[m = row tile's row l % 16][n = 4 (l / 16) .. + 3] of every tile pair
 #pragma unroll
   for (int mt = 0; mt < MW; ++mt) {
-    const int m = m0 + (mw * MW + mt) * 16 + c;
+    int m = m0 + (mw * MW + mt) * 16 + c;
     if (m >= M) continue;
+    if constexpr (MOE == 1) m += moe_row0;                 // the grouped row
+    if constexpr (MOE == 2) m = ma.perm[moe_row0 + m];     // (token, k)
 #pragma unroll
     for (int nt = 0; nt < (SWIGLU ? NT / 2 : NT); ++nt) {
       const int n = n0 + nt * 16 + 4 * g;
@@ -785,7 +814,36 @@ static int launch_wide(const void* A, const void* W, void* C, int M, int N, int 
     }
   }
   hipLaunchKernelGGL(kernel, grid, dim3(512), lds_bytes, stream, (const bf16_t*)A, (const bf16_t*)W, (TC*)C, M, N, K,
-                     up_offset, qa);
+                     up_offset, qa, MoeTileArgs{});
+  SA_LAUNCH_CHECK();
+  return 0;
+}
+
+// the experts' products: tiles of MOE_WIDE_ROWS grouped rows, 128 weight rows a workgroup (64 gates and their ups)
+constexpr int MOE_WIDE_MW = 2;
+constexpr int MOE_WIDE_ROWS = 64 * MOE_WIDE_MW;
+
+template <typename TC, int EPI, int MOE>
+static int launch_wide_moe(const void* A, const void* W, void* C, int N, int K, int up_offset, int max_tiles,
+                           const QkvRopeArgs& qa, const MoeTileArgs& ma, hipStream_t stream) {
+  constexpr int MW = MOE_WIDE_MW, NT = 8, NB = 4;
+  constexpr int COLS = EPI == EPI_SWIGLU ? 8 * NT : 16 * NT;
+  constexpr size_t lds_bytes = (size_t)NB * (64 * MW + 16 * NT) * 128;
+  static_assert(lds_bytes <= 160 * 1024, "the LDS of a compute unit");
+  dim3 grid((N + COLS - 1) / COLS, 1, max_tiles);
+  if (max_tiles < 1 || max_tiles > 65535) return SA_ERR_ARG;
+  auto kernel = gemm_wide_kernel<MW, NT, NB, TC, EPI, 1, MOE>;
+  static bool allowed[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return SA_ERR_ARG;
+  if (!allowed[dev]) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (e != hipSuccess) return (int)e;
+    allowed[dev] = true;
+  }
+  hipLaunchKernelGGL(kernel, grid, dim3(512), lds_bytes, stream, (const bf16_t*)A, (const bf16_t*)W, (TC*)C, 0, N, K,
+                     up_offset, qa, ma);
   SA_LAUNCH_CHECK();
   return 0;
 }
@@ -1077,4 +1135,26 @@ extern "C" int sa_gemm_bf16_qkv_rope(const void* A, const void* W, void* Q, cons
   if (takes_wide<bf16_t, EPI_QKV_ROPE>(M, 0, K, 1)) return pick_wide<bf16_t, EPI_QKV_ROPE>(A, W, Q, M, (Hq + 2 * Hk) * D, K, 0, 1, qa, stream);
   if (!takes_skinny<bf16_t, EPI_QKV_ROPE>(M, 0, qa)) return pick_mid<bf16_t, EPI_QKV_ROPE>(A, W, Q, M, (Hq + 2 * Hk) * D, K, 0, 1, qa, stream);
   return pick_skinny<bf16_t, EPI_QKV_ROPE>(A, W, Q, M, (Hq + 2 * Hk) * D, K, 0, 1, qa, stream);
+}
+
+extern "C" int sa_moe_wide_tile_rows() { return MOE_WIDE_ROWS; }
+
+// The two products of routed experts over tiles of sa_moe_wide_tile_rows() grouped rows (lists built by
+// sa_moe_experts with products = 0; max_tiles: the grid's worst case, rows / tile_rows + E).  bf16; d and F
+// multiples of 64 (whole stages of K).
+//   gate/up: h [T, d] gathered by perm / top, Wgu [2, E, F, d] -> act [rows, F] = gate(gate, up)
+//   down:    act [rows, F], Wd [E, d, F] -> yk [T top, d] fp32 at row perm[r]
+extern "C" int sa_moe_wide(const void* h, const void* Wgu, const void* Wd, void* act, float* yk, int E, int d, int F,
+                           int max_tiles, const int* offsets, const int* perm, const int* tile_expert,
+                           const int* tile_row0, const int* num_tiles, int top, int gate_kind, float gate_limit,
+                           hipStream_t stream) {
+  if (E <= 0 || d <= 0 || F <= 0 || (d & 63) || (F & 63) || top <= 0) return SA_ERR_ARG;
+  if (gate_kind < 0 || gate_kind >= SA_GATE_KINDS || (long long)E * F > 0x7fffffffLL) return SA_ERR_ARG;
+  QkvRopeArgs qa = {};
+  qa.gate_kind = gate_kind;
+  qa.gate_limit = gate_limit;
+  const MoeTileArgs ma = {offsets, perm, tile_expert, tile_row0, num_tiles, top};
+  int rc = launch_wide_moe<bf16_t, EPI_SWIGLU, 1>(h, Wgu, act, F, d, E * F, max_tiles, qa, ma, stream);
+  if (rc != 0) return rc;
+  return launch_wide_moe<float, EPI_PLAIN, 2>(act, Wd, yk, d, F, 0, max_tiles, qa, ma, stream);
 }

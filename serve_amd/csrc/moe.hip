@@ -522,6 +522,27 @@ extern "C" int sa_moe_experts(const void* h, int act_dtype, int* ids, const void
   return 0;
 }
 
+// Only the grouping (and, with logits, the routing): the lists for products that another library runs over tiles of
+// `tile_rows` grouped rows.  ints: as for sa_moe_experts, with max_tiles = sa_moe_max_tiles(T top, E).
+extern "C" int sa_moe_group(int* ids, int* ints, int T, int top, int E, int tile_rows, const float* logits, int ldz,
+                            float* wts, int over_all, float wscale, hipStream_t stream) {
+  if (T <= 0) return 0;
+  const long long n = (long long)T * top;
+  if (E <= 0 || top <= 0 || tile_rows < 16 || n > 0x3fffffffLL) return SA_ERR_ARG;
+  if (logits && (T > MOE_ROUTE_INSIDE || !wts || ldz < E || top > E)) return SA_ERR_ARG;
+  const int max_tiles = sa_moe_max_tiles((int)n, E);
+  int* offsets = ints;
+  int* cursor = offsets + E + 1;
+  int* perm = cursor + E;
+  int* tile_expert = perm + n;
+  int* tile_row0 = tile_expert + max_tiles;
+  int* num_tiles = tile_row0 + max_tiles;
+  hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), 0, stream, ids, (int)n, E, tile_rows, offsets, cursor, perm,
+                     tile_expert, tile_row0, num_tiles, logits, ldz, ids, wts, top, over_all, wscale);
+  SA_LAUNCH_CHECK();
+  return 0;
+}
+
 extern "C" int sa_moe_combine(const float* yk, const float* wts, const void* shared, int shared_dtype, int parts,
                               const float* sg, int ldz, float* y, int T, int top, int d, hipStream_t stream) {
   if (T <= 0) return 0;

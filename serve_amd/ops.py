@@ -632,6 +632,15 @@ def moe_route(logits: torch.Tensor, experts: int, top: int, ids: torch.Tensor, w
 
 
 MOE_ROUTE_INSIDE = 16      # up to this many tokens the experts' call does the routing itself (one kernel less)
+MOE_WIDE_MIN_ROWS = 1024   # more (token, k) rows than this take the products with both operands through LDS
+
+
+def moe_wide_available(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor) -> bool:
+    """bf16, widths that are whole stages of 64, and the gates' and ups' matrices one behind the other in memory
+    (`w_up` is the second half of the tensor whose first half is `w_gate`: [2, E, F, d])."""
+    E, F, d = w_gate.shape
+    return (h.dtype == torch.bfloat16 and d % 64 == 0 and F % 64 == 0 and _aligned16(h, w_gate, w_down)
+            and w_up.data_ptr() == w_gate.data_ptr() + w_gate.numel() * w_gate.element_size())
 
 
 def moe_experts(h: torch.Tensor, ids: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor,
@@ -657,6 +666,21 @@ def moe_experts(h: torch.Tensor, ids: torch.Tensor, w_gate: torch.Tensor, w_up: 
     tiles = int(lib.sa_moe_max_tiles(c_int(n), c_int(E)))
     ints = torch.empty(2 * E + 1 + n + 2 * tiles + 1, dtype=torch.int32, device=h.device)
     act = torch.empty((n, F), dtype=h.dtype, device=h.device)
+    if n > MOE_WIDE_MIN_ROWS and logits is None and moe_wide_available(h, w_gate, w_up, w_down):
+        # prompt portions: the grouping here, the two products over tiles of 128 rows with both operands through LDS
+        wide = load_library("gemm_mfma")
+        rows = int(wide.sa_moe_wide_tile_rows())
+        _ret(lib.sa_moe_group(_ptr(ids), _ptr(ints), c_int(T), c_int(top), c_int(E), c_int(rows), c_void_p(0), c_int(0),
+                              c_void_p(0), c_int(0), c_float(1.0), _stream()), "moe_group")
+        base, o = ints.data_ptr(), 4
+        offsets, perm = base, base + o * (2 * E + 1)
+        tile_expert = perm + o * n
+        tile_row0, num_tiles = tile_expert + o * tiles, tile_expert + o * 2 * tiles
+        _ret(wide.sa_moe_wide(_ptr(h), _ptr(w_gate), _ptr(w_down), _ptr(act), _ptr(yk), c_int(E), c_int(d), c_int(F),
+                              c_int(-(-n // rows) + E), c_void_p(offsets), c_void_p(perm), c_void_p(tile_expert),
+                              c_void_p(tile_row0), c_void_p(num_tiles), c_int(top), c_int(GATES[gate]), c_float(limit),
+                              _stream()), "moe_wide")
+        return yk
     ldz = 0
     if logits is not None:
         _check(T <= MOE_ROUTE_INSIDE and logits.dtype == torch.float32 and logits.dim() == 2 and logits.shape[0] == T

@@ -104,8 +104,9 @@ class RoutedExperts(Part):
         rows = [router] + ([tensors["shared.sg"].to(router.dtype)] if self.shared_gate else [])
         self.w_router = torch.cat(rows, dim=0).contiguous()              # the shared expert's gate rides along
         dt = rt.dtype
-        self.w_gate = torch.stack([tensors[f"e{e}.gate"].to(dt) for e in range(E)]).contiguous()
-        self.w_up = torch.stack([tensors[f"e{e}.up"].to(dt) for e in range(E)]).contiguous()
+        # (gates and ups in one tensor [2, E, F, d]: the kernel for many rows finds an expert's ups E F rows behind its gates)
+        gate_up = torch.stack([torch.stack([tensors[f"e{e}.{m}"].to(dt) for e in range(E)]) for m in ("gate", "up")]).contiguous()
+        self.w_gate, self.w_up = gate_up[0], gate_up[1]
         self.w_down = torch.stack([tensors[f"e{e}.down"].to(dt) for e in range(E)]).contiguous()
         if self.shared is not None:
             self.shared.load({"gate_proj.weight": tensors["shared.gate"], "up_proj.weight": tensors["shared.up"],

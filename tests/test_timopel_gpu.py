@@ -571,3 +571,40 @@ def test_steps_with_prompt_portions_replayed_from_graphs(tmp_path, dtype):
             seq.append(tok)
             compared += 1
     assert compared > 3 * count
+
+
+@pytest.mark.parametrize("gate,limit", [("silu", 0.0), ("clamped_swish", 0.8)])
+@pytest.mark.parametrize("T,d,F,E,top", [(700, 128, 192, 5, 2), (300, 64, 64, 9, 4), (2048, 256, 128, 6, 1)])
+def test_experts_of_many_rows_with_both_operands_through_lds(T, d, F, E, top, gate, limit):
+    """More than 1,024 (token, k) rows in bf16 with widths that are multiples of 64 and the gates' and ups' matrices in
+    one tensor: tiles of 128 grouped rows; experts with no row, with a few, and with several tiles of rows."""
+    from serve_amd import ops
+    torch.manual_seed(T + E)
+    h = torch.randn(T, d, device="cuda").bfloat16()
+    wgu = (torch.randn(2, E, F, d, device="cuda") * 0.1).bfloat16()
+    wd = (torch.randn(E, d, F, device="cuda") * 0.1).bfloat16()
+    assert T * top > ops.MOE_WIDE_MIN_ROWS and ops.moe_wide_available(h, wgu[0], wgu[1], wd)
+    ids = torch.stack([torch.randperm(E, device="cuda")[:top] for _ in range(T)]).int().contiguous()
+    if top < E:
+        ids[ids == E - 1] = 0 if top == 1 else ids[ids == E - 1]          # (top 1: the last expert gets no row at all)
+    ids[: T // 2, 0] = ids[0, 0]                                          # one expert with many tiles of rows
+    if top > 1:
+        ids[: T // 2, 1:] = ids[0, 1:]
+    yk = torch.full((T * top, d), float("nan"), dtype=torch.float32, device="cuda")
+    ops.moe_experts(h, ids, wgu[0], wgu[1], wd, yk, gate=gate, limit=limit)
+    assert torch.isfinite(yk).all(), "a row was not written"
+    # the same through the kernels for few rows, slice by slice
+    ref = torch.empty_like(yk)
+    for t0 in range(0, T, 200):
+        n = min(200, T - t0)
+        ops.moe_experts(h[t0: t0 + n].contiguous(), ids[t0: t0 + n].contiguous(), wgu[0], wgu[1], wd,
+                        ref[t0 * top: (t0 + n) * top], gate=gate, limit=limit)
+    assert torch.allclose(yk, ref, atol=2e-2, rtol=2e-2), f"max diff {(yk - ref).abs().max().item():.3g}"
+    hd = h.double().cpu()
+    for t in (0, 1, T // 2 - 1, T // 2, T - 1):
+        for k in range(top):
+            e = int(ids[t, k])
+            g, u = hd[t] @ wgu[0, e].double().cpu().t(), hd[t] @ wgu[1, e].double().cpu().t()
+            a = (tp.clamped_swish_gate(g, u, limit) if gate == "clamped_swish" else g * torch.sigmoid(g) * u).bfloat16().double()
+            want = a @ wd[e].double().cpu().t()
+            assert torch.allclose(yk[t * top + k].double().cpu(), want, atol=2e-2, rtol=1e-2)
